@@ -19,6 +19,7 @@ CSRC = os.path.dirname(os.path.abspath(__file__))
 # sources per activation type: each has matrix-core kernels of its own
 # (host/: the step executor and its way into the vendor's matrix library, host code that calls the kernels' entry points)
 COMMON_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "moe.hip", "sampling.hip", "delta_rule.hip", "head_gemm.hip",
+                  "lightning.hip",
                   "host/engine.cpp", "host/vendor.cpp"]
 SOURCES = {
     "float32": COMMON_SOURCES + ["gemm_f32.hip", "attention_f32.hip"],

@@ -112,6 +112,19 @@ __device__ __forceinline__ float gate_fn(float x, int kind) {
   return x;
 }
 
+// A gated pair with a limit (limit > 0): the gate's input is capped from above at the limit, the other factor is held
+// within +-limit and raised by one, f(min(g, limit)) * (clamp(u, -limit, limit) + 1); limit 0: f(g) * u.
+__device__ __forceinline__ float gated_pair(float g, float u, int kind, float limit) {
+  if (limit > 0.f) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit) + 1.0f;
+  }
+  return gate_fn(g, kind) * u;
+}
+// The limit that the products' launchers put into their argument blocks (tq_set_pair_limit sets it; 0: none).  It is
+// read on the host when a launch is made and travels as a kernel argument from there on.
+extern float tq_pair_limit_host;
+
 #define TQ_LAUNCH_CHECK()                        \
   do {                                           \
     hipError_t e__ = hipGetLastError();          \

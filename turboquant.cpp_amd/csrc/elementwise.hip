@@ -245,6 +245,14 @@ TQ_API int tq_add_rmsnorm(float* x, const float* delta, int S, int64_t delta_str
   return 0;
 }
 
+// The limit of gated pairs that the next launches of products and of gated_act take (common.h: gated_pair); 0: none.
+float tq_pair_limit_host = 0.f;
+TQ_API int tq_set_pair_limit(float limit) {
+  if (!(limit >= 0.f)) return TQ_ERR_BAD_ARG;
+  tq_pair_limit_host = limit;
+  return 0;
+}
+
 // ---------------------------------------------------------------- the gate of a gated pair, applied afterwards
 // out[m][n] = f(gu[m][n]) * gu[m][N + n]: for a pair of products that came out of one plain product over the two
 // matrices laid one behind the other (a library's, which has no such epilogue).  gu is float32 with row stride ld.
@@ -252,7 +260,8 @@ TQ_API int tq_add_rmsnorm(float* x, const float* delta, int S, int64_t delta_str
 // alone, an activation behind a plain product; gate < 0: f is the identity, a change of type)
 template <bool VEC>
 __global__ __launch_bounds__(256) void gated_act_kernel(const float* __restrict__ gp, int64_t ldg, const float* __restrict__ up,
-                                                        int64_t ldu, act_t* __restrict__ out, int N, int gate) {
+                                                        int64_t ldu, act_t* __restrict__ out, int N, int gate,
+                                                        float limit) {
   const float* row = gp + (size_t)blockIdx.y * ldg;
   const float* urow = up ? up + (size_t)blockIdx.y * ldu : nullptr;
   act_t* dst = out + (size_t)blockIdx.y * N;
@@ -260,15 +269,25 @@ __global__ __launch_bounds__(256) void gated_act_kernel(const float* __restrict_
     const int n = (blockIdx.x * 256 + threadIdx.x) * 4;
     if (n >= N) return;
     f32x4 g = load4f(row + n);
-    if (gate >= 0) g = f32x4{gate_fn(g.x, gate), gate_fn(g.y, gate), gate_fn(g.z, gate), gate_fn(g.w, gate)};
-    if (urow) g *= load4f(urow + n);
+    if (gate >= 0 && urow && limit > 0.f) {
+      const f32x4 u = load4f(urow + n);
+      g = f32x4{gated_pair(g.x, u.x, gate, limit), gated_pair(g.y, u.y, gate, limit), gated_pair(g.z, u.z, gate, limit),
+                gated_pair(g.w, u.w, gate, limit)};
+    } else {
+      if (gate >= 0) g = f32x4{gate_fn(g.x, gate), gate_fn(g.y, gate), gate_fn(g.z, gate), gate_fn(g.w, gate)};
+      if (urow) g *= load4f(urow + n);
+    }
     store4(dst + n, g);
   } else {
     const int n = blockIdx.x * 256 + threadIdx.x;
     if (n >= N) return;
     float g = row[n];
-    if (gate >= 0) g = gate_fn(g, gate);
-    if (urow) g *= urow[n];
+    if (gate >= 0 && urow && limit > 0.f) {
+      g = gated_pair(g, urow[n], gate, limit);
+    } else {
+      if (gate >= 0) g = gate_fn(g, gate);
+      if (urow) g *= urow[n];
+    }
     dst[n] = from_f32<act_t>(g);
   }
 }
@@ -281,9 +300,11 @@ static int launch_gated_act(const float* g, int64_t ldg, const float* u, int64_t
   const bool vec = N % 4 == 0 && ldg % 4 == 0 && ((uintptr_t)g % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
                    (!u || (ldu % 4 == 0 && ((uintptr_t)u % 16) == 0));
   if (vec)
-    hipLaunchKernelGGL(gated_act_kernel<true>, dim3((N / 4 + 255) / 256, M), dim3(256), 0, st, g, ldg, u, ldu, (act_t*)out, N, gate);
+    hipLaunchKernelGGL(gated_act_kernel<true>, dim3((N / 4 + 255) / 256, M), dim3(256), 0, st, g, ldg, u, ldu, (act_t*)out, N, gate,
+                       tq_pair_limit_host);
   else
-    hipLaunchKernelGGL(gated_act_kernel<false>, dim3((N + 255) / 256, M), dim3(256), 0, st, g, ldg, u, ldu, (act_t*)out, N, gate);
+    hipLaunchKernelGGL(gated_act_kernel<false>, dim3((N + 255) / 256, M), dim3(256), 0, st, g, ldg, u, ldu, (act_t*)out, N, gate,
+                       tq_pair_limit_host);
   TQ_LAUNCH_CHECK();
   return 0;
 }
@@ -327,6 +348,28 @@ TQ_API int tq_gate_rows(const void* o, const float* gate, int64_t ldg, void* out
   return 0;
 }
 
+// out[m][h hd + i] = f(gate[m][h]) * o[m][h hd + i]: one number per head and token gates the head's whole output.
+__global__ __launch_bounds__(256) void gate_heads_kernel(const act_t* __restrict__ o, const float* __restrict__ gate, int64_t ldg,
+                                                         act_t* __restrict__ out, int heads, int hd, int kind) {
+  const int m = blockIdx.y, N = heads * hd;
+  for (int n = blockIdx.x * 256 + threadIdx.x; n < N; n += gridDim.x * 256)
+    out[(size_t)m * N + n] = from_f32<act_t>(to_f32(o[(size_t)m * N + n]) * gate_fn(gate[(size_t)m * ldg + n / hd], kind));
+}
+
+TQ_API int tq_gate_heads(const void* o, const float* gate, int64_t ldg, void* out, int M, int heads, int hd, int kind,
+                         hipStream_t st) {
+  if (M <= 0 || heads <= 0 || hd <= 0) return 0;
+  if (kind < 0 || kind >= TQ_GATE_COUNT || ldg < heads) return TQ_ERR_BAD_ARG;
+  const int N = heads * hd;
+  for (int r = 0; r < M; r += 65535) {
+    const int rows = M - r < 65535 ? M - r : 65535;
+    hipLaunchKernelGGL(gate_heads_kernel, dim3((N + 1023) / 1024 < 1 ? 1 : (N + 1023) / 1024, rows), dim3(256), 0, st,
+                       (const act_t*)o + (size_t)r * N, gate + (size_t)r * ldg, ldg, (act_t*)out + (size_t)r * N, heads, hd, kind);
+  }
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
 // ---------------------------------------------------------------- RMS norm of a run of columns, written several times
 // out[t][c * Rp + i] = in[t][i] / sqrt(mean_i(in[t][i]^2) + eps) * w[i] for i < R, 0 for R <= i < Rp, for the copies
 // c = 0 .. copies - 1: the normed latent of an attention that keeps one compressed row per position, laid where the
@@ -355,6 +398,44 @@ TQ_API int tq_latent_norm(const float* in, int64_t ld_in, const void* w, int wty
   TQ_DISPATCH_W(wtype, {
     hipLaunchKernelGGL(latent_norm_kernel<W>, dim3((T + 3) / 4), dim3(256), 0, st, in, ld_in, (const W*)w, eps, out, ld_out,
                        copies, R, Rp, T);
+  });
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// The same with `lead` columns that are not normed: in[t][R .. R + lead) pass as they are and come first in every copy,
+// out[t][c * Rp + i] = in[t][R + i] for i < lead, the normed in[t][i - lead] for lead <= i < lead + R, 0 up to Rp (a
+// latent whose row also carries a part of the key that is rotated later and shared by all heads).  OUT_ACT: the copies
+// are written in the activation type (a normed row that feeds the next product).
+template <class W, class O>
+__global__ __launch_bounds__(256) void lead_norm_kernel(const float* __restrict__ in, int64_t ld_in, const W* __restrict__ w,
+                                                        float eps, O* __restrict__ out, int64_t ld_out, int copies, int R,
+                                                        int lead, int Rp, int T) {
+  const int t = blockIdx.x * 4 + threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
+  if (t >= T) return;
+  const float* row = in + (size_t)t * ld_in;
+  float ss = 0.f;
+  for (int i = lane; i < R; i += TQ_WAVE) ss += row[i] * row[i];
+  ss = wave_sum(ss);
+  const float rs = 1.0f / sqrtf(ss / (float)R + eps);
+  for (int i = lane; i < Rp; i += TQ_WAVE) {
+    const float v = i < lead ? row[R + i] : i < lead + R ? row[i - lead] * rs * to_f32(w[i - lead]) : 0.f;
+    for (int c = 0; c < copies; ++c) out[(size_t)t * ld_out + (size_t)c * Rp + i] = from_f32<O>(v);
+  }
+}
+
+TQ_API int tq_lead_norm(const float* in, int64_t ld_in, const void* w, int wtype, float eps, void* out, int out_is_act,
+                        int64_t ld_out, int copies, int R, int lead, int Rp, int T, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (R < 1 || lead < 0 || Rp < R + lead || copies < 1 || ld_in < R + lead || ld_out < (int64_t)copies * Rp || !w)
+    return TQ_ERR_BAD_ARG;
+  TQ_DISPATCH_W(wtype, {
+    if (out_is_act)
+      hipLaunchKernelGGL((lead_norm_kernel<W, act_t>), dim3((T + 3) / 4), dim3(256), 0, st, in, ld_in, (const W*)w, eps,
+                         (act_t*)out, ld_out, copies, R, lead, Rp, T);
+    else
+      hipLaunchKernelGGL((lead_norm_kernel<W, float>), dim3((T + 3) / 4), dim3(256), 0, st, in, ld_in, (const W*)w, eps,
+                         (float*)out, ld_out, copies, R, lead, Rp, T);
   });
   TQ_LAUNCH_CHECK();
   return 0;
@@ -422,14 +503,14 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(const float* __restr
                                      int bt_stride, const float* __restrict__ inv_freq, int pairing, int rot,
                                      act_t* __restrict__ q_out, act_t* __restrict__ k_pool,
                                      act_t* __restrict__ v_pool, int page_size, int64_t page_stride, int nh,
-                                     int nkv, int hd, int write_kv, int spb) {
+                                     int nkv, int hd, int write_kv, int spb, int64_t ld, float amp) {
   const int t = blockIdx.x;
   const int wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
   const int heads = nh + 2 * nkv;       // 0..nh-1 query heads, then key heads, then value heads
   const int s0 = blockIdx.y * spb + wave, s1 = min(blockIdx.y * spb + spb, heads);
   if (s0 >= s1) return;
   const int pos = positions[t];
-  const float* src_t = qkv + (size_t)t * heads * hd;
+  const float* src_t = qkv + (size_t)t * ld;
   act_t* q_t = q_out + (size_t)t * nh * hd;
   act_t *k_t = nullptr, *v_t = nullptr;      // the token's row of kv head 0 in its page
   if (write_kv && s1 > nh) {
@@ -445,6 +526,8 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(const float* __restr
     const float theta = (float)pos * inv_freq[i];
     float sn, cs;
     sincosf(theta, &sn, &cs);
+    sn *= amp;      // (an amplitude of 1 changes no bit)
+    cs *= amp;
     const int ia = pairing == 0 ? i : 2 * i;
     const int ib = pairing == 0 ? i + half : 2 * i + 1;
     for (int s = s0; s < rot_end; s += 4) {
@@ -472,6 +555,94 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(const float* __restr
   }
 }
 
+// The same with a norm behind the rotation: every rotated query and key head is divided by its root mean square over
+// its first norm_dim values, x / sqrt(mean(x^2) + eps), no weights (heads laid out wider hold zeros behind them).  A wave
+// takes a head at a time: a lane keeps the sines and cosines of its pairs (up to four: heads of up to 512), sums the
+// squares of what it has turned, and scales as it stores.
+template <int BIAS>
+__global__ __launch_bounds__(256) void rope_norm_kv_write_kernel(const float* __restrict__ qkv, const void* __restrict__ bias,
+                                     const int* __restrict__ positions,
+                                     const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
+                                     int bt_stride, const float* __restrict__ inv_freq, int pairing, int rot,
+                                     act_t* __restrict__ q_out, act_t* __restrict__ k_pool,
+                                     act_t* __restrict__ v_pool, int page_size, int64_t page_stride, int nh,
+                                     int nkv, int hd, int write_kv, int spb, int64_t ld, float amp, float eps,
+                                     int norm_dim) {
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
+  const int heads = nh + 2 * nkv;
+  const int s0 = blockIdx.y * spb + wave, s1 = min(blockIdx.y * spb + spb, heads);
+  if (s0 >= s1) return;
+  const int pos = positions[t];
+  const float* src_t = qkv + (size_t)t * ld;
+  act_t* q_t = q_out + (size_t)t * nh * hd;
+  act_t *k_t = nullptr, *v_t = nullptr;
+  if (write_kv && s1 > nh) {
+    const int page = block_table[(size_t)seq_of_token[t] * bt_stride + pos / page_size];
+    const int row = pos % page_size;
+    k_t = k_pool + (size_t)page * page_stride + (size_t)row * hd;
+    v_t = v_pool + (size_t)page * page_stride + row;
+  }
+  const int rot_end = write_kv ? min(s1, nh + nkv) : min(s1, nh);
+  const size_t kv_head_stride = (size_t)page_size * hd;
+  const int half = rot / 2;
+  float cs[4], sn[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = lane + TQ_WAVE * j;
+    cs[j] = 1.f;
+    sn[j] = 0.f;
+    if (i < half) {
+      sincosf((float)pos * inv_freq[i], &sn[j], &cs[j]);
+      sn[j] *= amp;
+      cs[j] *= amp;
+    }
+  }
+  for (int s = s0; s < rot_end; s += 4) {
+    const float* src = src_t + (size_t)s * hd;
+    act_t* dst = s < nh ? q_t + (size_t)s * hd : k_t + (size_t)(s - nh) * kv_head_stride;
+    float ra[4], rb[4], ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = lane + TQ_WAVE * j;
+      ra[j] = rb[j] = 0.f;
+      if (i < half) {
+        const int ia = pairing == 0 ? i : 2 * i;
+        const int ib = pairing == 0 ? i + half : 2 * i + 1;
+        const float a = src[ia] + bias_elem<BIAS>(bias, (size_t)s * hd + ia);
+        const float b = src[ib] + bias_elem<BIAS>(bias, (size_t)s * hd + ib);
+        ra[j] = a * cs[j] - b * sn[j];
+        rb[j] = a * sn[j] + b * cs[j];
+        ss = fmaf(ra[j], ra[j], ss);
+        ss = fmaf(rb[j], rb[j], ss);
+      }
+    }
+    for (int i = rot + lane; i < hd; i += TQ_WAVE) {
+      const float v = src[i] + bias_elem<BIAS>(bias, (size_t)s * hd + i);
+      ss = fmaf(v, v, ss);
+    }
+    const float rs = 1.0f / sqrtf(wave_sum(ss) / (float)norm_dim + eps);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = lane + TQ_WAVE * j;
+      if (i < half) {
+        dst[pairing == 0 ? i : 2 * i] = from_f32<act_t>(ra[j] * rs);
+        dst[pairing == 0 ? i + half : 2 * i + 1] = from_f32<act_t>(rb[j] * rs);
+      }
+    }
+    for (int i = rot + lane; i < hd; i += TQ_WAVE)
+      dst[i] = from_f32<act_t>((src[i] + bias_elem<BIAS>(bias, (size_t)s * hd + i)) * rs);
+  }
+  if (write_kv != 1) return;
+  for (int s = s0; s < s1; s += 4) {
+    if (s < nh + nkv) continue;
+    const float* src = src_t + (size_t)s * hd;
+    act_t* col = v_t + (size_t)(s - nh - nkv) * kv_head_stride;
+    for (int i = lane; i < hd; i += TQ_WAVE)
+      col[(size_t)i * page_size] = from_f32<act_t>(src[i] + bias_elem<BIAS>(bias, (size_t)s * hd + i));
+  }
+}
+
 // The values of runs of tokens, one run per sequence (tokens cu_seqlens[b] .. of sequence b lie at positions
 // start[b] ..): a workgroup takes 64 positions that share a page (grid (chunks, nkv, B)), turns their rows
 // [position][hd] into [hd][position] in LDS and writes every dimension's positions 16 bytes at a time, where the
@@ -485,7 +656,7 @@ __global__ __launch_bounds__(256) void v_write_tile_kernel(const float* __restri
                                                            const int* __restrict__ start,
                                                            const int* __restrict__ block_table, int bt_stride,
                                                            act_t* __restrict__ v_pool, int page_size,
-                                                           int64_t page_stride, int nh, int nkv, int hd) {
+                                                           int64_t page_stride, int nh, int nkv, int hd, int64_t ld) {
   extern __shared__ __attribute__((aligned(16))) unsigned char vt_raw[];
   act_t* ts = (act_t*)vt_raw;                        // [hd][VT_POS + VEC]
   constexpr int TS = VT_POS + VEC;
@@ -495,9 +666,8 @@ __global__ __launch_bounds__(256) void v_write_tile_kernel(const float* __restri
   const int lo = max(P0, st), hi = min(P0 + VT_POS, st + n);
   if (lo >= hi) return;
   const int wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
-  const int heads = nh + 2 * nkv;
-  const float* src0 = qkv + ((size_t)(t0 + lo - st) * heads + nh + nkv + h) * hd;      // value row of position lo
-  const size_t row_stride = (size_t)heads * hd;
+  const float* src0 = qkv + (size_t)(t0 + lo - st) * ld + (size_t)(nh + nkv + h) * hd;      // value row of position lo
+  const size_t row_stride = (size_t)ld;
   const size_t bias0 = (size_t)(nh + nkv + h) * hd;      // the bias of this value head
   if (hd % 4 == 0) {        // 16 bytes of a row per thread and turn, all of a thread's loads on their way at once
     const int q4 = hd / 4, total = (hi - lo) * q4;
@@ -536,13 +706,19 @@ __global__ __launch_bounds__(256) void v_write_tile_kernel(const float* __restri
 // cu_seqlens, slots, start (null, or [B + 1], [B], [B] with max_new the longest run): the tokens as runs of
 // consecutive positions, one per sequence; given for whole prompts, they let the values go by tiles.
 // bias (null, or [(nh + 2 nkv) * hd] of bias_type): added to qkv as it is read, for a product that left it out.
-TQ_API int tq_rope_kv_write(const float* qkv, const void* bias, int bias_type, const int* positions, const int* seq_of_token,
-                            const int* block_table, int bt_stride, const float* inv_freq, int pairing, int rot,
-                            void* q_out, void* k_pool, void* v_pool, int page_size, int64_t page_stride, int T,
-                            int nh, int nkv, int hd, int write_kv, const int* cu_seqlens, const int* slots,
-                            const int* start, int B, int max_new, hipStream_t st) {
+// ld: floats between the rows of two tokens in qkv (at least (nh + 2 nkv) * hd: the rows may be runs of columns of a
+// wider product).  amp: a factor on every sine and cosine (1: none).  norm_eps > 0: the rotated query and key heads are
+// divided by their root mean square over norm_dim values (rope_norm_kv_write_kernel; heads of up to 512).
+TQ_API int tq_rope_kv_write_ex(const float* qkv, int64_t ld, const void* bias, int bias_type, const int* positions,
+                               const int* seq_of_token, const int* block_table, int bt_stride, const float* inv_freq,
+                               int pairing, int rot, float amp, float norm_eps, int norm_dim, void* q_out, void* k_pool,
+                               void* v_pool, int page_size, int64_t page_stride, int T, int nh, int nkv, int hd, int write_kv,
+                               const int* cu_seqlens, const int* slots, const int* start, int B, int max_new,
+                               hipStream_t st) {
   if (T <= 0) return 0;
   if (rot < 0 || rot > hd || (rot & 1) || (pairing != 0 && pairing != 1)) return TQ_ERR_BAD_ARG;
+  if (ld < (int64_t)(nh + 2 * nkv) * hd || norm_eps < 0.f) return TQ_ERR_BAD_ARG;
+  if (norm_eps > 0.f && (norm_dim < 1 || norm_dim > hd || rot > 512)) return TQ_ERR_BAD_ARG;
   if (bias && bias_type != TQ_F32 && bias_type != TQ_BF16) return TQ_ERR_BAD_ARG;
   constexpr int VEC = 16 / (int)sizeof(act_t);
   const size_t vt_shmem = (size_t)hd * (VT_POS + VEC) * sizeof(act_t);
@@ -556,9 +732,18 @@ TQ_API int tq_rope_kv_write(const float* qkv, const void* bias, int bias_type, c
   if ((heads + spb - 1) / spb > 65535) return TQ_ERR_UNSUPPORTED;
   const int bias_kind = !bias ? 0 : bias_type == TQ_F32 ? 1 : 2;
 #define TQ_ROPE_LAUNCH(BIAS)                                                                                          \
-  hipLaunchKernelGGL(rope_kv_write_kernel<BIAS>, dim3(T, (heads + spb - 1) / spb), dim3(256), 0, st, qkv, bias,       \
-                     positions, seq_of_token, block_table, bt_stride, inv_freq, pairing, rot, (act_t*)q_out,          \
-                     (act_t*)k_pool, (act_t*)v_pool, page_size, page_stride, nh, nkv, hd, write_kv, spb)
+  do {                                                                                                                \
+    if (norm_eps > 0.f)                                                                                               \
+      hipLaunchKernelGGL(rope_norm_kv_write_kernel<BIAS>, dim3(T, (heads + spb - 1) / spb), dim3(256), 0, st, qkv,    \
+                         bias, positions, seq_of_token, block_table, bt_stride, inv_freq, pairing, rot,               \
+                         (act_t*)q_out, (act_t*)k_pool, (act_t*)v_pool, page_size, page_stride, nh, nkv, hd,          \
+                         write_kv, spb, ld, amp, norm_eps, norm_dim);                                                 \
+    else                                                                                                              \
+      hipLaunchKernelGGL(rope_kv_write_kernel<BIAS>, dim3(T, (heads + spb - 1) / spb), dim3(256), 0, st, qkv, bias,   \
+                         positions, seq_of_token, block_table, bt_stride, inv_freq, pairing, rot, (act_t*)q_out,      \
+                         (act_t*)k_pool, (act_t*)v_pool, page_size, page_stride, nh, nkv, hd, write_kv, spb, ld,      \
+                         amp);                                                                                        \
+  } while (0)
   if (bias_kind == 0) TQ_ROPE_LAUNCH(0);
   else if (bias_kind == 1) TQ_ROPE_LAUNCH(1);
   else TQ_ROPE_LAUNCH(2);
@@ -572,7 +757,7 @@ TQ_API int tq_rope_kv_write(const float* qkv, const void* bias, int bias_type, c
                                 (int)vt_shmem);                                                                       \
     hipLaunchKernelGGL((v_write_tile_kernel<VEC, BIAS>), dim3((max_new + VT_POS - 1) / VT_POS + 1, nkv, B), dim3(256), \
                        vt_shmem, st, qkv, bias, cu_seqlens, slots, start, block_table, bt_stride, (act_t*)v_pool,     \
-                       page_size, page_stride, nh, nkv, hd);                                                          \
+                       page_size, page_stride, nh, nkv, hd, ld);                                                      \
   } while (0)
     if (bias_kind == 0) TQ_VT_LAUNCH(0);
     else if (bias_kind == 1) TQ_VT_LAUNCH(1);
@@ -581,6 +766,16 @@ TQ_API int tq_rope_kv_write(const float* qkv, const void* bias, int bias_type, c
     TQ_LAUNCH_CHECK();
   }
   return 0;
+}
+
+TQ_API int tq_rope_kv_write(const float* qkv, const void* bias, int bias_type, const int* positions, const int* seq_of_token,
+                            const int* block_table, int bt_stride, const float* inv_freq, int pairing, int rot,
+                            void* q_out, void* k_pool, void* v_pool, int page_size, int64_t page_stride, int T,
+                            int nh, int nkv, int hd, int write_kv, const int* cu_seqlens, const int* slots,
+                            const int* start, int B, int max_new, hipStream_t st) {
+  return tq_rope_kv_write_ex(qkv, (int64_t)(nh + 2 * nkv) * hd, bias, bias_type, positions, seq_of_token, block_table,
+                             bt_stride, inv_freq, pairing, rot, 1.0f, 0.f, hd, q_out, k_pool, v_pool, page_size, page_stride,
+                             T, nh, nkv, hd, write_kv, cu_seqlens, slots, start, B, max_new, st);
 }
 
 // ---------------------------------------------------------------- sum of expert outputs

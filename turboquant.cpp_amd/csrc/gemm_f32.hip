@@ -46,6 +46,7 @@ struct F32GemmArgs {
   int64_t ldc;
   int M, N, K;
   int gate;                // activation of the gated pair
+  float limit;             // of the gated pair (gated_pair in common.h); 0: none
 };
 
 __device__ __forceinline__ float f32_bias_at(const F32GemmArgs& g, int n) {
@@ -185,7 +186,7 @@ __global__ __launch_bounds__(256) void gemm_f32_tile_kernel(F32GemmArgs g, int k
           continue;
         }
         float x = acc[i][j][v] + f32_bias_at(g, n);
-        if (DUAL) x = gate_fn(x, g.gate) * acc2[i][j][v];
+        if (DUAL) x = gated_pair(x, acc2[i][j][v], g.gate, g.limit);
         g.out[(size_t)m * g.ldc + n] = x;
       }
     }
@@ -377,7 +378,7 @@ __global__ __launch_bounds__(256) void gemm_f32_stream_kernel(F32GemmArgs g, int
           if (DUAL) dst[(size_t)gridDim.z * g.M * g.N + (size_t)m * ld + nn] = acc2[c][t][v];
         } else {
           float x = acc[c][t][v] + f32_bias_at(g, nn);
-          if (DUAL) x = gate_fn(x, g.gate) * acc2[c][t][v];
+          if (DUAL) x = gated_pair(x, acc2[c][t][v], g.gate, g.limit);
           dst[(size_t)m * ld + nn] = x;
         }
       }
@@ -396,7 +397,7 @@ __global__ void gemm_f32_reduce_kernel(F32GemmArgs g, const float* __restrict__ 
     if (dual) y += part[(size_t)(S + z) * g.M * g.N + i];
   }
   x += f32_bias_at(g, n);
-  if (dual) x = gate_fn(x, g.gate) * y;
+  if (dual) x = gated_pair(x, y, g.gate, g.limit);
   g.out[(size_t)m * g.ldc + n] = x;
 }
 __global__ void gemm_f32_bias_kernel(F32GemmArgs g) {
@@ -440,7 +441,7 @@ TQ_API int tq_gemm_f32(const void* a, int64_t lda, const int* a_rows, int a_gath
     return TQ_ERR_UNSUPPORTED;
   if (gate < 0 || gate >= TQ_GATE_COUNT) return TQ_ERR_BAD_ARG;
   F32GemmArgs g{(const float*)a, lda, a_rows, a_gather, (const float*)w, (const float*)w2, group_stride, tile_group,
-                n_tiles, bias, bias_type, (float*)out, ldc, M, N, K, gate};
+                n_tiles, bias, bias_type, (float*)out, ldc, M, N, K, gate, tq_pair_limit_host};
   const bool dual = w2 != nullptr;
   const bool grouped = tile_group != nullptr;
   if (keep_runs && (dual || grouped || a_rows || ldc != N)) return TQ_ERR_BAD_ARG;

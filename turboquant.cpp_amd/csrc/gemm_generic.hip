@@ -30,6 +30,7 @@ struct GemmArgs {
   int64_t ldc;
   int M, N, K;
   int gate;                // activation of the gated pair
+  float limit;             // of the gated pair (gated_pair in common.h); 0: none
 };
 
 template <class W, int TM, bool DUAL, bool OUT_ACT>
@@ -107,7 +108,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmArgs g) {
       if (n >= g.N) continue;
       float v = acc[i][j];
       if (g.bias) v += g.bias_type == TQ_F32 ? ((const float*)g.bias)[n] : to_f32(((const bf16_t*)g.bias)[n]);
-      if (DUAL) v = gate_fn(v, g.gate) * acc2[i][j];
+      if (DUAL) v = gated_pair(v, acc2[i][j], g.gate, g.limit);
       if (OUT_ACT)
         ((act_t*)g.out)[(size_t)m * g.ldc + n] = from_f32<act_t>(v);
       else
@@ -139,7 +140,7 @@ TQ_API int tq_gemm_generic(const void* a, int64_t lda, const int* a_rows, int a_
   if (K <= 0 || (tile_rows != 16 && tile_rows != 64)) return TQ_ERR_BAD_ARG;
   if ((N + BN - 1) / BN > 65535) return TQ_ERR_UNSUPPORTED;
   if (gate < 0 || gate >= TQ_GATE_COUNT) return TQ_ERR_BAD_ARG;
-  GemmArgs g{(const act_t*)a, lda, a_rows, a_gather, w, w2, group_stride, tile_group, n_tiles, bias, bias_type, out, ldc, M, N, K, gate};
+  GemmArgs g{(const act_t*)a, lda, a_rows, a_gather, w, w2, group_stride, tile_group, n_tiles, bias, bias_type, out, ldc, M, N, K, gate, tq_pair_limit_host};
   TQ_DISPATCH_W(wtype, {
     if (tile_rows == 16)
       launch<W, 1>(g, w2 != nullptr, out_is_act != 0, st);

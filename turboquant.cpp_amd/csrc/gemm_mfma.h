@@ -29,6 +29,7 @@ struct MfmaGemmArgs {
   int gate;                 // activation of the gated pair
   int group_ratio;          // tile kernel: row tiles per entry of tile_group and unit of n_tiles (0 or 1: one)
   int act1;                 // a plain product (no w2, k not split): 0, or 1 + the activation its result passes before it is stored
+  float limit;              // of the gated pair (gated_pair in common.h); 0: none
 };
 
 // For bytes that are read once (a matrix streamed past a few rows): a load that tells the caches so.  Measured on

@@ -170,7 +170,7 @@ __device__ __forceinline__ void stream_body(MfmaGemmArgs g, int tile_n, int tile
       if (on >= g.N || om >= g.M) continue;
       if (g.a_rows && g.a_rows[om] < 0) continue;
       float o = s + bias_at(g, on);
-      if (DUAL) o = gate_fn(o, g.gate) * s2;
+      if (DUAL) o = gated_pair(o, s2, g.gate, g.limit);
       store_out<OUT_ACT>(g, om, on, o);
     }
     return;
@@ -188,7 +188,7 @@ __device__ __forceinline__ void stream_body(MfmaGemmArgs g, int tile_n, int tile
         if (m >= g.M) continue;
         if (g.a_rows && g.a_rows[m] < 0) continue;
         float o = acc[t][mt][v] + b;
-        if (DUAL) o = gate_fn(o, g.gate) * acc2[t][mt][v];
+        if (DUAL) o = gated_pair(o, acc2[t][mt][v], g.gate, g.limit);
         store_out<OUT_ACT>(g, m, n, o);
       }
   }
@@ -518,7 +518,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
         if (m >= g.M) continue;
         if (g.a_rows && g.a_rows[m] < 0) continue;
         float o = acc[mi][ni][v] + b;
-        if (DUAL) o = gate_fn(o, g.gate) * acc2[mi][ni][v];
+        if (DUAL) o = gated_pair(o, acc2[mi][ni][v], g.gate, g.limit);
         store_out<OUT_ACT>(g, m, n, o);
       }
   }
@@ -659,7 +659,7 @@ __global__ __launch_bounds__(1024) void gemm_ring_kernel(MfmaGemmArgs g) {
     if (m >= g.M) continue;
     if (g.a_rows && g.a_rows[m] < 0) continue;
     if (DUAL) {
-      if (na < g.N) store_out<OUT_ACT>(g, m, na, gate_fn(acc[v] + ba, g.gate) * acc2[v]);
+      if (na < g.N) store_out<OUT_ACT>(g, m, na, gated_pair(acc[v] + ba, acc2[v], g.gate, g.limit));
     } else {
       if (na < g.N) store_out<OUT_ACT>(g, m, na, acc[v] + ba);
       if (nb < g.N) store_out<OUT_ACT>(g, m, nb, acc2[v] + bb);
@@ -867,7 +867,7 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
   if (splits > 1 && (int64_t)(splits - 1) * k_per >= K) return TQ_ERR_BAD_ARG;
   MfmaGemmArgs g{(const bf16_t*)a, lda, a_rows, a_gather, (const bf16_t*)w, (const bf16_t*)w2, group_stride,
                  tile_group, n_tiles, bias, bias_type, out, ldc, M, N, K, splits > 1 ? k_per : K, (int64_t)M * ldc, gate, 1,
-                 alone ? gate + 1 : 0};
+                 alone ? gate + 1 : 0, tq_pair_limit_host};
   int rc = 0;
   if (tile_group) {
     if (tile_rows == 16) {
@@ -967,7 +967,7 @@ TQ_API int tq_gemm_mfma_pair(const int64_t* d1, const int64_t* d2, int splits2, 
     if (((uintptr_t)p[0] | (uintptr_t)p[4] | (uintptr_t)p[5]) % 16 != 0) return TQ_ERR_BAD_ARG;
     g[i] = MfmaGemmArgs{(const bf16_t*)p[0], p[1], (const int*)p[2], (int)p[3], (const bf16_t*)p[4], (const bf16_t*)p[5],
                         p[6], (const int*)p[7], (const int*)p[8], (const void*)p[9], (int)p[10], (void*)p[11], p[12],
-                        M, N, K, K, 0, (int)p[18], 1};
+                        M, N, K, K, 0, (int)p[18], 1, 0, tq_pair_limit_host};
     if (g[i].gate < 0 || g[i].gate >= TQ_GATE_COUNT) return TQ_ERR_BAD_ARG;
     dual[i] = p[5] != 0;
     out_act[i] = p[13] != 0;

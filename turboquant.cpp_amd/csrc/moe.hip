@@ -38,7 +38,8 @@ __device__ __forceinline__ void load4(const bf16_t* p, float* w) {
 template <class W, int TG, int RW>
 __global__ __launch_bounds__(256) void router_logits_kernel(const float* __restrict__ x, const W* __restrict__ wr,
                                                             const W* __restrict__ shared_w, int rows, int E,
-                                                            float* __restrict__ logits, int T, int H) {
+                                                            float* __restrict__ logits, int T, int H,
+                                                            const float* __restrict__ bias) {
   extern __shared__ __attribute__((aligned(16))) float xs[];      // [TG][Hp]
   const int Hp = (H + 511) / 512 * 512;
   const int t0 = blockIdx.x * TG;
@@ -132,7 +133,8 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float* __restr
 #pragma unroll
       for (int k = 0; k < TG; ++k) {
         const float v = wave_sum(s[r][k]);
-        if (lane == 0 && k < nt && idx + r < rows) logits[(size_t)(t0 + k) * rows + e[r]] = v;
+        if (lane == 0 && k < nt && idx + r < rows)      // (a bias per expert, not for the shared expert's gate row)
+          logits[(size_t)(t0 + k) * rows + e[r]] = bias && e[r] < E ? v + bias[e[r]] : v;
       }
   }
 }
@@ -252,7 +254,7 @@ __global__ __launch_bounds__(256) void router_select_kernel(const float* __restr
 }
 
 static int launch_router_logits(const float* x, const void* wr, const void* shared_w, int wtype, int E,
-                                float* logits, int T, int H, hipStream_t st) {
+                                float* logits, int T, int H, hipStream_t st, const float* bias = nullptr) {
   int tg = RT;
   const size_t hp = ((size_t)H + 511) / 512 * 512;      // a token's row in LDS
   while (tg > 1 && (size_t)tg * hp * sizeof(float) > 32 * 1024) tg /= 2;   // small enough for several workgroups per CU
@@ -272,7 +274,7 @@ static int launch_router_logits(const float* x, const void* wr, const void* shar
       (void)hipFuncSetAttribute((const void*)router_logits_kernel<W, TGV, RWV>,                                           \
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);                                  \
     hipLaunchKernelGGL((router_logits_kernel<W, TGV, RWV>), dim3(groups, row_groups), dim3(256), shmem, st, x,      \
-                       (const W*)wr, (const W*)shared_w, rows, E, logits, T, H);                                    \
+                       (const W*)wr, (const W*)shared_w, rows, E, logits, T, H, bias);                              \
   } while (0)
 #define TQ_ROUTER_RW(TGV)          \
   do {                             \
@@ -299,19 +301,27 @@ static int groups_ok(int E, int topk, int groups, int keep) {
   return groups >= 1 && groups <= 256 && E % groups == 0 && keep >= 1 && keep <= groups && topk <= keep * (E / groups);
 }
 
-TQ_API int tq_router_topk_grouped(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk,
-                                  int renorm, int groups, int keep, int* ids, float* weights, float* shared_gate,
-                                  float* logits, int T, int H, hipStream_t st) {
+// bias (null, or float [E]): added to the experts' logits before the choice.
+TQ_API int tq_router_topk_biased(const float* x, const void* wr, const void* shared_w, const float* bias, int wtype, int E,
+                                 int topk, int renorm, int groups, int keep, int* ids, float* weights, float* shared_gate,
+                                 float* logits, int T, int H, hipStream_t st) {
   if (T <= 0) return 0;
   if (topk < 1 || topk > 64 || topk > E || E > 8192) return TQ_ERR_UNSUPPORTED;
   if (!groups_ok(E, topk, groups, keep)) return TQ_ERR_BAD_ARG;
-  const int rc = launch_router_logits(x, wr, shared_w, wtype, E, logits, T, H, st);
+  const int rc = launch_router_logits(x, wr, shared_w, wtype, E, logits, T, H, st, bias);
   if (rc) return rc;
   const int rows = E + (shared_w ? 1 : 0);
   hipLaunchKernelGGL(router_select_kernel, dim3((T + 3) / 4), dim3(256), (size_t)4 * E * sizeof(float), st, logits,
                      rows, E, topk, renorm, groups, keep, ids, weights, shared_gate, T);
   TQ_LAUNCH_CHECK();
   return 0;
+}
+
+TQ_API int tq_router_topk_grouped(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk,
+                                  int renorm, int groups, int keep, int* ids, float* weights, float* shared_gate,
+                                  float* logits, int T, int H, hipStream_t st) {
+  return tq_router_topk_biased(x, wr, shared_w, nullptr, wtype, E, topk, renorm, groups, keep, ids, weights, shared_gate,
+                               logits, T, H, st);
 }
 
 TQ_API int tq_router_topk(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk,
@@ -650,16 +660,16 @@ TQ_API int tq_moe_align(const int* ids, int n_pairs, int E, int topk, int unit, 
 // several workgroups order the pairs (the same order).  logits: scratch of T * (E + 1) floats (T * E without a shared
 // gate vector); what it holds afterwards means nothing.
 // groups, keep: the choice within the best `keep` of `groups` groups of experts (1, 1: among all).
-TQ_API int tq_route_grouped(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk, int renorm,
-                            int groups, int keep, int* ids, float* weights, float* shared_gate, float* logits, int unit,
-                            int cap, int* sorted_token, int* pair_slot, int* tile_expert, int* n_tiles, int T, int H,
-                            hipStream_t st) {
+TQ_API int tq_route_biased(const float* x, const void* wr, const void* shared_w, const float* bias, int wtype, int E,
+                           int topk, int renorm, int groups, int keep, int* ids, float* weights, float* shared_gate,
+                           float* logits, int unit, int cap, int* sorted_token, int* pair_slot, int* tile_expert,
+                           int* n_tiles, int T, int H, hipStream_t st) {
   if (T <= 0) return 0;
   if (!groups_ok(E, topk, groups, keep)) return TQ_ERR_BAD_ARG;
   const size_t shmem = ((size_t)(AW + 1) * E + (size_t)AW * topk + (size_t)AW * E) * 4;
   if (T > AW || shmem > 64 * 1024) {
-    const int rc = tq_router_topk_grouped(x, wr, shared_w, wtype, E, topk, renorm, groups, keep, ids, weights, shared_gate,
-                                          logits, T, H, st);
+    const int rc = tq_router_topk_biased(x, wr, shared_w, bias, wtype, E, topk, renorm, groups, keep, ids, weights,
+                                         shared_gate, logits, T, H, st);
     if (rc) return rc;
     // once the experts are chosen the logits are done with: the order by several workgroups keeps its table there
     const int n = T * topk;
@@ -672,7 +682,7 @@ TQ_API int tq_route_grouped(const float* x, const void* wr, const void* shared_w
   if (topk < 1 || topk > 64 || topk > E || E > 8192) return TQ_ERR_UNSUPPORTED;
   const int n_pairs = T * topk;
   if (unit < 1 || cap % unit != 0 || cap < n_pairs + (E < n_pairs ? E : n_pairs) * (unit - 1)) return TQ_ERR_BAD_ARG;
-  const int rc = launch_router_logits(x, wr, shared_w, wtype, E, logits, T, H, st);
+  const int rc = launch_router_logits(x, wr, shared_w, wtype, E, logits, T, H, st, bias);
   if (rc) return rc;
   if (T == 1) {      // one wave: its barriers cost nothing
     const size_t shmem1 = ((size_t)2 * E + topk + E) * 4;
@@ -687,6 +697,14 @@ TQ_API int tq_route_grouped(const float* x, const void* wr, const void* shared_w
                      renorm, groups, keep, ids, weights, shared_gate, T, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles);
   TQ_LAUNCH_CHECK();
   return 0;
+}
+
+TQ_API int tq_route_grouped(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk, int renorm,
+                            int groups, int keep, int* ids, float* weights, float* shared_gate, float* logits, int unit,
+                            int cap, int* sorted_token, int* pair_slot, int* tile_expert, int* n_tiles, int T, int H,
+                            hipStream_t st) {
+  return tq_route_biased(x, wr, shared_w, nullptr, wtype, E, topk, renorm, groups, keep, ids, weights, shared_gate, logits,
+                         unit, cap, sorted_token, pair_slot, tile_expert, n_tiles, T, H, st);
 }
 
 TQ_API int tq_route(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk, int renorm,

@@ -90,6 +90,20 @@ _SIGNATURES = {
     "tq_delta_out": [_c_ptr, _c_ptr, _c_ptr, _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int,
                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
     "tq_sample_topp": [_c_ptr, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "tq_set_pair_limit": [_c_f32],
+    "tq_gate_heads": [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "tq_lead_norm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_f32, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int,
+                     _c_ptr],
+    "tq_rope_kv_write_ex": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_f32,
+                            _c_f32, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int,
+                            _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
+    "tq_router_topk_biased": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr,
+                              _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
+    "tq_route_biased": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
+                        _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
+    "tq_lightning_scan": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_ptr,
+                          _c_ptr],
+    "tq_lightning_out": [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_int, _c_f32, _c_ptr, _c_int, _c_int, _c_ptr],
 }
 # entry points that only one of the two libraries has
 _OPTIONAL = {
@@ -204,7 +218,8 @@ _KIND = {"gemm": "matmul", "gemm_mfma": "matmul", "gemm_f32": "matmul", "gemm_pa
          "gated_act": "matmul", "attention": "attn", "attention_mfma": "attn", "attention_f32": "attn",
          "router_topk": "moe", "route": "moe", "moe_align": "moe", "moe_combine": "moe",
          "delta_prep": "attn", "delta_scan": "attn", "delta_out": "attn", "delta_decode": "attn",
-         "head_gemm": "matmul", "latent_norm": "attn", "gate_rows": "attn"}
+         "head_gemm": "matmul", "latent_norm": "attn", "gate_rows": "attn", "gate_heads": "attn",
+         "lightning_scan": "attn", "lightning_out": "attn"}
 
 
 def profile_begin() -> None:
@@ -436,9 +451,13 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torc
                   inv_freq: torch.Tensor, pairing: int, rotary_dim: int, k_pages: torch.Tensor | None,
                   v_pages: torch.Tensor | None, layer_offset: int, page_size: int, page_stride: int,
                   num_heads: int, num_kv_heads: int, head_dim: int, act, runs: dict | None = None,
-                  bias: torch.Tensor | None = None) -> torch.Tensor:
+                  bias: torch.Tensor | None = None, amplitude: float = 1.0, norm_eps: float | None = None,
+                  norm_dim: int | None = None) -> torch.Tensor:
     """Rotates queries and keys, returns the queries [T, nh*hd] and writes keys and values into the pages.
-    ``bias`` [width] is added to ``qkv`` as it is read, for a product that left its bias out.
+    ``bias`` [width] is added to ``qkv`` as it is read, for a product that left its bias out.  ``qkv`` may be the first
+    columns of the rows of a wider tensor.  ``amplitude``: a factor on every sine and cosine.  ``norm_eps``: behind the
+    rotation every query and key head is divided by its root mean square over its first ``norm_dim`` values (all of the
+    head by default; heads laid out wider hold zeros behind them), without weights.
     ``k_pages``/``v_pages`` are the flat page pools of the cache group (None: nothing is written, for a
     layer that reads another layer's cache); ``layer_offset`` is the layer's offset inside a page.  ``runs``
     (as for ``attention``) describes the tokens as one run of consecutive positions per sequence; with it the
@@ -446,9 +465,14 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torc
     k = "rope_kv_write"
     T = positions.numel()
     width = (num_heads + 2 * num_kv_heads) * head_dim
-    _check(qkv, k, "qkv", torch.float32, (T, width))
+    _need(isinstance(qkv, torch.Tensor) and qkv.is_cuda and qkv.dtype == torch.float32 and tuple(qkv.shape) == (T, width)
+          and qkv.stride(1) == 1 and qkv.stride(0) >= width, k,
+          lambda: f"qkv must be float32 [{T}, {width}] on the GPU with unit stride along its rows")
+    _need(k_pages is None or head_dim % 4 != 0 or (qkv.stride(0) % 4 == 0 and qkv.data_ptr() % 16 == 0), k,
+          "rows of qkv must start at multiples of 16 bytes")
     if bias is not None:
         _check(bias, k, "bias", tuple(_WTYPE), (width,))
+    _need(norm_eps is None or (norm_eps > 0 and rotary_dim <= 512), k, "a norm behind the rotation needs a positive eps and at most 512 rotated values")
     _check(positions, k, "positions", torch.int32, (T,))
     _check(seq_of_token, k, "seq_of_token", torch.int32, (T,))
     _check(block_table, k, "block_table", torch.int32)
@@ -474,11 +498,12 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torc
         _check(slots, k, "slots", torch.int32, (B,))
         _check(start, k, "start", torch.int32, (B,))
         _need(int(runs["max_end"]) <= block_table.shape[1] * page_size, k, "positions reach beyond the page table")
-    _run(k, library(act).tq_rope_kv_write(_ptr(qkv), _ptr(bias), _WTYPE[bias.dtype] if bias is not None else 0,
-                                          _ptr(positions), _ptr(seq_of_token), _ptr(block_table),
-                                          block_table.shape[1], _ptr(inv_freq), pairing, rotary_dim, _ptr(q), kp, vp,
-                                          page_size, page_stride, T, num_heads, num_kv_heads, head_dim, int(write),
-                                          _ptr(cu), _ptr(slots), _ptr(start), B, max_new, _stream()))
+    _run(k, library(act).tq_rope_kv_write_ex(_ptr(qkv), qkv.stride(0), _ptr(bias), _WTYPE[bias.dtype] if bias is not None else 0,
+                                             _ptr(positions), _ptr(seq_of_token), _ptr(block_table),
+                                             block_table.shape[1], _ptr(inv_freq), pairing, rotary_dim, float(amplitude),
+                                             float(norm_eps or 0.0), int(norm_dim or head_dim), _ptr(q), kp, vp,
+                                             page_size, page_stride, T, num_heads, num_kv_heads, head_dim, int(write),
+                                             _ptr(cu), _ptr(slots), _ptr(start), B, max_new, _stream()))
     return q
 
 
@@ -758,9 +783,10 @@ def _use_f32(act, a: torch.Tensor, w: torch.Tensor, K: int, gstride: int) -> boo
 def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None, w2: torch.Tensor | None = None,
          out_act: bool = False, a_rows: torch.Tensor | None = None, tile_group: torch.Tensor | None = None,
          n_tiles: torch.Tensor | None = None, tile_rows: int | None = None, gather: bool = True,
-         partial_sums: bool = False, activation: str = "silu", act_alone: bool = False) -> torch.Tensor:
+         partial_sums: bool = False, activation: str = "silu", act_alone: bool = False,
+         pair_limit: float | None = None) -> torch.Tensor:
     """out[m, n] = sum_k a[row(m), k] * w[g, n, k]  (+ bias[n]);  with ``w2``: f(a w^T) * (a w2^T), f being the
-    ``activation`` (silu, gelu_tanh or relu2).  ``act_alone`` (a plain product, no ``w2``): f of the product, in the
+    ``activation`` (a name of GATES); with ``pair_limit`` L beside it: f(min(a w^T, L)) * (clamp(a w2^T, -L, L) + 1).  ``act_alone`` (a plain product, no ``w2``): f of the product, in the
     activation type: in the product's own epilogue where this library's matrix-core kernel runs it, else in a launch
     of its own behind it.
 
@@ -772,6 +798,16 @@ def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None
     k that the caller adds up in order, as the next norm does with a part's output; the kernel chooses S.
     """
     k = "gemm"
+    if pair_limit is not None:
+        # the launchers read the limit as they fill their argument blocks; from there on it is a kernel argument
+        _need(w2 is not None and pair_limit > 0, k, "a limit is for gated pairs and positive")
+        lib = library(act)
+        lib.tq_set_pair_limit(float(pair_limit))
+        try:
+            return gemm(a, w, act, bias=bias, w2=w2, out_act=out_act, a_rows=a_rows, tile_group=tile_group, n_tiles=n_tiles,
+                        tile_rows=tile_rows, gather=gather, partial_sums=partial_sums, activation=activation)
+        finally:
+            lib.tq_set_pair_limit(0.0)
     adt = ACT_DTYPES[dtype_name(act)]
     grouped = tile_group is not None
     M, N, K, tile_rows, gstride = _gemm_problem(k, a, w, act, bias, w2, out_act, a_rows, tile_group, n_tiles, tile_rows,
@@ -982,15 +1018,18 @@ def _expert_groups(k: str, E: int, top_k: int, groups) -> tuple[int, int]:
 
 
 def router_topk(x32: torch.Tensor, router: torch.Tensor, shared_scale: torch.Tensor | None, top_k: int,
-                renormalize: bool, act, groups: tuple[int, int] | None = None):
+                renormalize: bool, act, groups: tuple[int, int] | None = None, bias: torch.Tensor | None = None):
     """ids int32 [T, k], weights float32 [T, k], and sigmoid(x . shared_scale) float32 [T] (or None).
-    ``groups`` (count, keep): only experts of the ``keep`` groups with the largest best score can be chosen."""
+    ``groups`` (count, keep): only experts of the ``keep`` groups with the largest best score can be chosen.
+    ``bias`` float32 [E]: added to the experts' logits before the choice."""
     k = "router_topk"
     T, H, E, ids, weights, gate, logits = _router_outputs(k, x32, router, shared_scale, top_k)
     count, keep = _expert_groups(k, E, top_k, groups)
-    _run(k, library(act).tq_router_topk_grouped(_ptr(x32), _ptr(router), _ptr(shared_scale), _WTYPE[router.dtype], E, top_k,
-                                                int(bool(renormalize)), count, keep, _ptr(ids), _ptr(weights), _ptr(gate),
-                                                _ptr(logits), T, H, _stream()))
+    if bias is not None:
+        _check(bias, k, "bias", torch.float32, (E,))
+    _run(k, library(act).tq_router_topk_biased(_ptr(x32), _ptr(router), _ptr(shared_scale), _ptr(bias), _WTYPE[router.dtype], E,
+                                               top_k, int(bool(renormalize)), count, keep, _ptr(ids), _ptr(weights), _ptr(gate),
+                                               _ptr(logits), T, H, _stream()))
     return ids, weights, gate
 
 
@@ -1025,18 +1064,20 @@ def _align_outputs(T: int, topk: int, num_experts: int, unit: int, dev):
 
 
 def route(x32: torch.Tensor, router: torch.Tensor, shared_scale: torch.Tensor | None, top_k: int, renormalize: bool,
-          unit: int, act, groups: tuple[int, int] | None = None):
+          unit: int, act, groups: tuple[int, int] | None = None, bias: torch.Tensor | None = None):
     """``router_topk`` followed by ``moe_align`` in one call: (ids, weights, gate, sorted_token, pair_slot,
     tile_expert, n_tiles), with the same results; a handful of tokens takes one kernel less."""
     k = "route"
     T, H, E, ids, weights, gate, logits = _router_outputs(k, x32, router, shared_scale, top_k)
     _need(unit in (16, 32, 64, 128, 256), k, "unit must be 16, 32, 64, 128 or 256")
     count, keep = _expert_groups(k, E, top_k, groups)
+    if bias is not None:
+        _check(bias, k, "bias", torch.float32, (E,))
     cap, sorted_token, pair_slot, tile_expert, n_tiles = _align_outputs(T, top_k, E, unit, x32.device)
-    _run(k, library(act).tq_route_grouped(_ptr(x32), _ptr(router), _ptr(shared_scale), _WTYPE[router.dtype], E, top_k,
-                                          int(bool(renormalize)), count, keep, _ptr(ids), _ptr(weights), _ptr(gate),
-                                          _ptr(logits), unit, cap, _ptr(sorted_token), _ptr(pair_slot), _ptr(tile_expert),
-                                          _ptr(n_tiles), T, H, _stream()))
+    _run(k, library(act).tq_route_biased(_ptr(x32), _ptr(router), _ptr(shared_scale), _ptr(bias), _WTYPE[router.dtype], E, top_k,
+                                         int(bool(renormalize)), count, keep, _ptr(ids), _ptr(weights), _ptr(gate),
+                                         _ptr(logits), unit, cap, _ptr(sorted_token), _ptr(pair_slot), _ptr(tile_expert),
+                                         _ptr(n_tiles), T, H, _stream()))
     return ids, weights, gate, sorted_token, pair_slot, tile_expert, n_tiles
 
 
@@ -1371,6 +1412,83 @@ def head_gemm(a: torch.Tensor, w: torch.Tensor, act, out: torch.Tensor | None = 
     _run(k, library(act).tq_head_gemm(_ptr(a), _WTYPE[a.dtype], a.stride(0), _ptr(w), _WTYPE[w.dtype], _ptr(out), int(out_act),
                                       out.stride(0), _ptr(gate), gate.stride(0) if gate is not None else 0,
                                       _gate_code(k, activation), T, H, N, K, _stream()))
+    return out
+
+
+def gate_heads(o: torch.Tensor, gate: torch.Tensor, num_heads: int, activation: str, act) -> torch.Tensor:
+    """o[:, h * hd : (h + 1) * hd] *= f(gate[:, h]), in place: one number per head and token gates the head's whole output.
+    ``o`` [M, heads * hd] contiguous in the activation type, ``gate`` float32 [M, heads] whose rows may be runs of
+    columns of a wider tensor."""
+    k = "gate_heads"
+    _check(o, k, "o", ACT_DTYPES[dtype_name(act)])
+    M, N = o.shape
+    _need(num_heads >= 1 and N % num_heads == 0, k, lambda: f"{N} columns are not {num_heads} heads")
+    _need(isinstance(gate, torch.Tensor) and gate.is_cuda and gate.dtype == torch.float32 and tuple(gate.shape) == (M, num_heads)
+          and gate.stride(1) == 1, k, lambda: f"gate must be float32 [{M}, {num_heads}] on the GPU with unit stride along its rows")
+    _run(k, library(act).tq_gate_heads(_ptr(o), _ptr(gate), gate.stride(0), _ptr(o), M, num_heads, N // num_heads,
+                                       _gate_code(k, activation), _stream()))
+    return o
+
+
+def lead_norm(src: torch.Tensor, rank: int, weight: torch.Tensor, eps: float, copies: int, width: int, act,
+              out: torch.Tensor | None = None, out_act: bool = False) -> torch.Tensor:
+    """Rows ``src`` (float32 [T, rank + lead], a run of columns of a wider tensor allowed): the first ``rank`` columns
+    are RMS-normed with ``weight`` [rank], the ``lead`` columns behind them pass as they are; every copy in ``out``
+    [T, copies * width] holds the lead first, then the normed columns, then zeros up to ``width``.  ``out`` is float32, or
+    of the activation type with ``out_act``."""
+    k = "lead_norm"
+    _need(isinstance(src, torch.Tensor) and src.is_cuda and src.dtype == torch.float32 and src.dim() == 2 and src.stride(1) == 1,
+          k, "src must be float32 [T, n] on the GPU with unit stride along its rows")
+    T, lead = src.shape[0], src.shape[1] - rank
+    _need(rank >= 1 and lead >= 0 and width >= rank + lead and copies >= 1, k, "rank, lead and width do not fit")
+    _check(weight, k, "weight", tuple(_WTYPE), (rank,))
+    odt = ACT_DTYPES[dtype_name(act)] if out_act else torch.float32
+    if out is None:
+        out = torch.empty((T, copies * width), dtype=odt, device=src.device)
+    _need(out.is_cuda and out.dtype == odt and tuple(out.shape) == (T, copies * width) and out.stride(1) == 1, k,
+          lambda: f"out must be [{T}, {copies * width}] {odt} with unit stride along its rows")
+    _run(k, library(act).tq_lead_norm(_ptr(src), src.stride(0), _ptr(weight), _WTYPE[weight.dtype], float(eps), _ptr(out),
+                                      int(out_act), out.stride(0), copies, rank, lead, width, T, _stream()))
+    return out
+
+
+# ------------------------------------------------------------------ linear attention with a decay per head
+def lightning_scan(proj: torch.Tensor, decay: torch.Tensor, runs: dict, state: torch.Tensor, num_heads: int, head_dim: int,
+                   value_dim: int, act) -> torch.Tensor:
+    """The recurrence S <- decay_h S + k v^T, o = S^T q over the step's runs of tokens, from and into the sequences' rows
+    of ``state`` (float32 [slots, heads * dim * vdim]); ``proj`` float32 [T, >= 2 H D + 2 H V] holds q | k | v | gate
+    before their silu.  Returns o float32 [T, H * V]."""
+    k = "lightning_scan"
+    H, D, V = num_heads, head_dim, value_dim
+    _need(isinstance(proj, torch.Tensor) and proj.is_cuda and proj.dtype == torch.float32 and proj.dim() == 2
+          and proj.stride(1) == 1 and proj.shape[1] >= 2 * H * D + 2 * H * V, k,
+          lambda: f"proj must be float32 [T, >= {2 * H * D + 2 * H * V}] on the GPU with unit stride along its rows")
+    _check(decay, k, "decay", torch.float32, (H,))
+    _check(state, k, "state", torch.float32)
+    _need(state.dim() == 2 and state.shape[1] == H * D * V, k, lambda: f"state must be [slots, {H * D * V}]")
+    _need(D <= 256, k, lambda: f"a key width of {D} is beyond the 256 this kernel takes")
+    B = runs["slots"].numel()
+    _check(runs["cu_seqlens"], k, "cu_seqlens", torch.int32, (B + 1,))
+    _check(runs["slots"], k, "slots", torch.int32, (B,))
+    T = proj.shape[0]
+    o = torch.empty((T, H * V), dtype=torch.float32, device=proj.device)
+    _run(k, library(act).tq_lightning_scan(_ptr(proj), proj.stride(0), _ptr(decay), _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]),
+                                           _ptr(state), state.stride(0), B, H, D, V, _ptr(o), _stream()))
+    return o
+
+
+def lightning_out(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, act) -> torch.Tensor:
+    """rmsnorm(o) * weight * sigmoid(gate) in the activation type, the norm over a token's whole row (all heads together):
+    ``o`` float32 [T, N] contiguous, ``gate`` float32 [T, N] whose rows may be runs of columns of a wider tensor."""
+    k = "lightning_out"
+    _check(o, k, "o", torch.float32)
+    T, N = o.shape
+    _need(isinstance(gate, torch.Tensor) and gate.is_cuda and gate.dtype == torch.float32 and tuple(gate.shape) == (T, N)
+          and gate.stride(1) == 1, k, lambda: f"gate must be float32 [{T}, {N}] on the GPU with unit stride along its rows")
+    _check(weight, k, "weight", tuple(_WTYPE), (N,))
+    out = torch.empty((T, N), dtype=ACT_DTYPES[dtype_name(act)], device=o.device)
+    _run(k, library(act).tq_lightning_out(_ptr(o), _ptr(gate), gate.stride(0), _ptr(weight), _WTYPE[weight.dtype], float(eps),
+                                          _ptr(out), T, N, _stream()))
     return out
 
 

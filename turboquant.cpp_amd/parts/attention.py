@@ -15,6 +15,12 @@ j <= i only if i // n == j // n, chunks counted from position 0 of the sequence)
 than keys); ``separate_qkv`` (q, k, v and their biases are parameters of their own, joined when the part is prepared);
 ``sink`` (a learned number per head whose exponential joins the softmax's denominator: a score with no key and no value,
 neither scaled nor capped, counted once).
+``rotated_norm_eps`` (behind the rotation every query and key head is divided by its root mean square over the head, no
+weights: the cache holds the keys so normed); ``head_gate`` (a matrix [heads, hidden]: head h's output is multiplied by
+the sigmoid of row h's product with the layer's input, before the output product); ``shares_kv`` (the mixer has no key and
+value matrices: its schedule entry reads the cache of an earlier entry, with queries, window and everything else of its
+own); ``cache_window`` (what the cache keeps where that is more than the mixer's own window, because a later layer that
+reads this cache looks further back; None: everything).  A position part may scale its sines and cosines (``amplitude``).
 With ``separate_qkv`` the heads are laid out at a kernel width that is the larger of key and value width rounded up to
 16: the added rows and columns of the matrices are zeros, which change no score and no output, and every head size
 then runs on the matrix-core kernels of both libraries.
@@ -37,7 +43,17 @@ class GroupedQueryAttention(Part):
                  qkv_bias: bool = False, out_bias: bool = False, window: int | None = None,
                  scale: float | None = None, qk_norm_eps: float | None = None, score_cap: float | None = None,
                  distance_bias: bool = False, chunk: int | None = None, value_dim: int | None = None,
-                 separate_qkv: bool = False, sink: bool = False):
+                 separate_qkv: bool = False, sink: bool = False, rotated_norm_eps: float | None = None,
+                 head_gate: bool = False, shares_kv: bool = False, cache_window: int | None | str = "own"):
+        if (head_gate or shares_kv) and not separate_qkv:
+            raise ValueError("a gate per head and a cache shared with another layer need separate_qkv")
+        if rotated_norm_eps is not None and not rotated_norm_eps > 0:
+            raise ValueError(f"rotated_norm_eps must be positive, got {rotated_norm_eps}")
+        if cache_window != "own" and cache_window is not None and (window is None or cache_window < window):
+            raise ValueError(f"the cache must keep at least the mixer's own window {window}, got {cache_window}")
+        self.rotated_norm_eps, self.has_head_gate, self.shares_kv = rotated_norm_eps, head_gate, shares_kv
+        self.cache_window = window if cache_window == "own" else cache_window
+        self.gate_weight = None
         if num_heads % num_kv_heads:
             raise ValueError(f"num_heads {num_heads} is not a multiple of num_kv_heads {num_kv_heads}")
         if window is not None and window < 1:
@@ -75,11 +91,15 @@ class GroupedQueryAttention(Part):
     def param_specs(self):
         if self.separate_qkv:
             H, G, K, V, W = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim, self.hidden_size
-            specs = {"q_weight": ParamSpec((H * K, W)), "k_weight": ParamSpec((G * K, W)), "v_weight": ParamSpec((G * V, W)),
-                     "out_weight": ParamSpec((W, H * V))}
+            specs = {"q_weight": ParamSpec((H * K, W)), "out_weight": ParamSpec((W, H * V))}
+            if not self.shares_kv:
+                specs.update({"k_weight": ParamSpec((G * K, W)), "v_weight": ParamSpec((G * V, W))})
+            if self.has_head_gate:
+                specs["gate_weight"] = ParamSpec((H, W))
             if self.has_qkv_bias:
-                specs.update({"q_bias": ParamSpec((H * K,), role="bias"), "k_bias": ParamSpec((G * K,), role="bias"),
-                              "v_bias": ParamSpec((G * V,), role="bias")})
+                specs["q_bias"] = ParamSpec((H * K,), role="bias")
+                if not self.shares_kv:
+                    specs.update({"k_bias": ParamSpec((G * K,), role="bias"), "v_bias": ParamSpec((G * V,), role="bias")})
             if self.has_out_bias:
                 specs["out_bias"] = ParamSpec((W,), role="bias")
             if self.has_distance_bias:
@@ -126,11 +146,21 @@ class GroupedQueryAttention(Part):
         H, G, K, V = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
         if self.qk_norm_eps is not None and K != D:     # zeros behind the head's own values: they norm zeros to zeros
             self.q_norm, self.k_norm = (torch.cat([w, w.new_zeros(D - K)]) for w in (self.q_norm, self.k_norm))
-        self.qkv_weight = torch.cat([heads_padded(self.q_weight, H, K), heads_padded(self.k_weight, G, K),
-                                     heads_padded(self.v_weight, G, V)])
+        rows = [heads_padded(self.q_weight, H, K)]
+        if not self.shares_kv:
+            rows += [heads_padded(self.k_weight, G, K), heads_padded(self.v_weight, G, V)]
+        if self.has_head_gate:      # the gate's rows ride in the same product, filled up to a multiple of four rows
+            fill = -H % 4
+            rows += [self.gate_weight, self.gate_weight.new_zeros((fill, self.hidden_size))]
+        self.qkv_weight = torch.cat(rows).contiguous()
         if self.has_qkv_bias:
-            self.qkv_bias = torch.cat([heads_padded(self.q_bias, H, K), heads_padded(self.k_bias, G, K),
-                                       heads_padded(self.v_bias, G, V)])
+            bias = [heads_padded(self.q_bias, H, K)]
+            if not self.shares_kv:
+                bias += [heads_padded(self.k_bias, G, K), heads_padded(self.v_bias, G, V)]
+            if self.has_head_gate:
+                bias.append(bias[0].new_zeros((H + -H % 4,)))
+            self.qkv_bias = torch.cat(bias).contiguous()
+        self.gate_weight = None
         if V != D:
             out = self.out_weight.new_zeros((self.hidden_size, H, D))
             out[:, :, :V] = self.out_weight.view(self.hidden_size, H, V)
@@ -141,7 +171,7 @@ class GroupedQueryAttention(Part):
         return {"position": self.position}
 
     def cache_need(self) -> CacheNeed:
-        return CacheNeed(self.num_kv_heads, self.head_dim, self.window, chunk=self.chunk)
+        return CacheNeed(self.num_kv_heads, self.head_dim, self.cache_window, chunk=self.chunk)
 
     def state_need(self):
         return None
@@ -152,6 +182,8 @@ class GroupedQueryAttention(Part):
             return None
         if self.score_cap is not None or self.has_distance_bias or self.chunk is not None or self.separate_qkv or self.has_sink:
             return None                         # nor one with changed scores or chunks
+        if self.rotated_norm_eps is not None or getattr(self.position, "amplitude", 1.0) != 1.0:
+            return None
         table = self.position.table(self.qkv_weight.device)
         if table.dtype != torch.float32 or not table.is_contiguous() or table.numel() * 2 != self.position.rotary_dim:
             return None
@@ -175,6 +207,9 @@ class GroupedQueryAttention(Part):
 
     def forward(self, normed, ctx, entry):
         b, kv = ctx.batch, ctx.kv(entry)
+        amplitude = getattr(self.position, "amplitude", 1.0)
+        if self.rotated_norm_eps is not None or self.has_head_gate or self.shares_kv or amplitude != 1.0:
+            return self._forward_extended(normed, ctx, b, kv, amplitude)
         rope = (b.positions, b.slot_of_token, kv.table, self.position.table(ctx.device), self.position.pairing_code,
                 self.position.rotary_dim, kv.k_pages if kv.owns else None, kv.v_pages if kv.owns else None,
                 kv.layer_offset, kv.page_size, kv.page_stride, self.num_heads, self.num_kv_heads, self.head_dim, ctx.act)
@@ -188,4 +223,30 @@ class GroupedQueryAttention(Part):
         o = ops.attention(q, kv.k_pages, kv.v_pages, kv.layer_offset, b.positions, b.slot_of_token, kv.table,
                           kv.page_size, kv.page_stride, self.num_heads, self.num_kv_heads, self.head_dim,
                           self.window, self.scale, ctx.act, runs=b.runs(), **self._score_options())
+        return ops.gemm(o, self.out_weight, ctx.act, bias=self.out_bias, partial_sums=True)
+
+    def _forward_extended(self, normed, ctx, b, kv, amplitude):
+        """The forms with a norm behind the rotation, scaled sines and cosines, a gate per head or another layer's keys
+        and values: one product of the layer's input (q | k | v | gate rows), the rotation with its norm and the cache
+        write in one launch, attention, the gate, the output product."""
+        if kv.owns == self.shares_kv:
+            raise ValueError("an attention keeps a cache of its own exactly if it has keys and values of its own")
+        H, G, D = self.num_heads, 0 if self.shares_kv else self.num_kv_heads, self.head_dim
+        proj = ops.gemm(normed, self.qkv_weight, ctx.act, bias=self.qkv_bias)
+        width = (H + 2 * G) * D
+        qkv = proj[:, :width]
+        if self.qk_norm_eps is not None:
+            if proj.shape[1] != width:
+                raise ValueError("the norm of the heads before the rotation does not go with a gate per head")
+            ops.head_rmsnorm(qkv, self.q_norm, None if self.shares_kv else self.k_norm, self.qk_norm_eps, H, G, D, ctx.act,
+                             norm_dim=self.key_dim)
+        q = ops.rope_kv_write(qkv, b.positions, b.slot_of_token, kv.table, self.position.table(ctx.device),
+                              self.position.pairing_code, self.position.rotary_dim, kv.k_pages if kv.owns else None,
+                              kv.v_pages if kv.owns else None, kv.layer_offset, kv.page_size, kv.page_stride, H, G, D, ctx.act,
+                              runs=b.runs(), amplitude=amplitude, norm_eps=self.rotated_norm_eps, norm_dim=self.key_dim)
+        o = ops.attention(q, kv.k_pages, kv.v_pages, kv.layer_offset, b.positions, b.slot_of_token, kv.table,
+                          kv.page_size, kv.page_stride, H, self.num_kv_heads, D, self.window, self.scale, ctx.act,
+                          runs=b.runs(), **self._score_options())
+        if self.has_head_gate:
+            ops.gate_heads(o, proj[:, width:width + H], H, "sigmoid", ctx.act)
         return ops.gemm(o, self.out_weight, ctx.act, bias=self.out_bias, partial_sums=True)

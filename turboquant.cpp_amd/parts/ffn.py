@@ -8,7 +8,8 @@ Sparse (/root/reference/src/engine/tq_moe.c:600-1059): router logits in float32,
 winning ties, weights from a softmax; every chosen expert is the dense formula with its own matrices, summed
 with its weight in the order chosen; the shared expert, scaled by ``sigmoid(x . shared_scale)``, is added
 last.  ``renormalize`` false keeps the softmax over all experts un-normalised for the chosen ones; true is
-the reference's softmax over the chosen logits.  ``groups`` (count, keep): the experts form ``count`` equal groups of
+the reference's softmax over the chosen logits.  ``router_bias``: a number per expert is added to its logit before the
+choice.  ``pair_limit`` L: an expert is ``down(f(min(gate x, L)) * (clamp(up x, -L, L) + 1))``.  ``groups`` (count, keep): the experts form ``count`` equal groups of
 neighbours, a group's score is the largest score in it, and only experts of the ``keep`` best groups can be chosen.
 """
 from __future__ import annotations
@@ -86,7 +87,12 @@ class SparseMoE(Part):
 
     def __init__(self, hidden_size: int, num_experts: int, top_k: int, expert_size: int, shared_size: int = 0,
                  shared_gated: bool = True, renormalize: bool = False, activation: str = "silu",
-                 groups: tuple[int, int] | None = None):
+                 groups: tuple[int, int] | None = None, router_bias: bool = False, pair_limit: float | None = None):
+        if pair_limit is not None and not pair_limit > 0:
+            raise ValueError(f"pair_limit must be positive, got {pair_limit}")
+        if (router_bias or pair_limit is not None) and shared_size > 0:
+            raise ValueError("a router with a bias and experts with a limit come without a shared expert")
+        self.has_router_bias, self.pair_limit, self.router_bias = router_bias, pair_limit, None
         if not 1 <= top_k <= num_experts:
             raise ValueError(f"top_k {top_k} must be within 1..num_experts {num_experts}")
         if groups is not None:
@@ -109,6 +115,8 @@ class SparseMoE(Part):
         specs = {"router": ParamSpec((E, H), role="router"),
                  "expert_gate": ParamSpec((E, I, H)), "expert_up": ParamSpec((E, I, H)),
                  "expert_down": ParamSpec((E, H, I))}
+        if self.has_router_bias:
+            specs["router_bias"] = ParamSpec((E,), role="bias")
         if S > 0:
             specs.update({"shared_gate": ParamSpec((S, H)), "shared_up": ParamSpec((S, H)),
                           "shared_down": ParamSpec((H, S))})
@@ -117,14 +125,16 @@ class SparseMoE(Part):
         return specs
 
     def prepare(self, device, act):
+        if self.has_router_bias:     # it enters float arithmetic only
+            self.router_bias = self.router_bias.float().contiguous()
         if self.shared_size > 0:     # as in the dense part; the experts' products never leave this library's kernels
             self.shared_gate, self.shared_up = ops.side_by_side(self.shared_gate, self.shared_up)
 
     def native(self):
         from ..csrc import host_api
         w = host_api.weight
-        if self.groups is not None:      # the executor chooses among all experts
-            return None
+        if self.groups is not None or self.has_router_bias or self.pair_limit is not None:
+            return None                  # the executor chooses among all experts, by logits without a bias, for plain pairs
         return host_api.MoeFfnDesc(self.hidden_size, self.num_experts, self.top_k, self.expert_size, self.shared_size,
                                    int(self.renormalize), ops.GATES[self.activation], w(self.router),
                                    w(self.shared_scale if self.shared_gated else None), w(self.expert_gate), w(self.expert_up),
@@ -136,7 +146,8 @@ class SparseMoE(Part):
                                     **({} if self.expert_size % 8 == 0 else {"w_behind": self.expert_down}))
         route = lambda: ops.route(normed32, self.router, self.shared_scale if self.shared_gated else None,
                                   self.top_k, self.renormalize, unit, ctx.act,
-                                  **({} if self.groups is None else {"groups": self.groups}))
+                                  **({} if self.groups is None else {"groups": self.groups}),
+                                  **({} if self.router_bias is None else {"bias": self.router_bias}))
         if self.shared_size > 0 and T <= 16 and unit == 16:
             # a handful of tokens: the shared expert's two products ride in the launches of the routed experts'
             _, weights, gate, sorted_token, pair_slot, tile_expert, n_tiles = route()
@@ -170,7 +181,8 @@ class SparseMoE(Part):
         _, weights, gate, sorted_token, pair_slot, tile_expert, n_tiles = route()
         rows = ops.expert_product_rows(unit, T * self.top_k, self.num_experts)
         h = ops.gemm(normed, self.expert_gate, ctx.act, w2=self.expert_up, out_act=True, a_rows=sorted_token,
-                     tile_group=tile_expert, n_tiles=n_tiles, tile_rows=rows, activation=self.activation)
+                     tile_group=tile_expert, n_tiles=n_tiles, tile_rows=rows, activation=self.activation,
+                     **({} if self.pair_limit is None else {"pair_limit": self.pair_limit}))
         y = ops.gemm(h, self.expert_down, ctx.act, a_rows=sorted_token, tile_group=tile_expert, n_tiles=n_tiles,
                      tile_rows=rows, gather=False)
         if side is not None:

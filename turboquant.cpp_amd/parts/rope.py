@@ -13,6 +13,8 @@ partial, with per-pair factors) is another table.
 """
 from __future__ import annotations
 
+import math
+
 import numpy as np
 import torch
 
@@ -24,6 +26,8 @@ PAIRINGS = {"half": 0, "interleaved": 1}
 @register_part("position", "rope")
 class RotaryEncoding(Part):
     graph_safe = True
+    amplitude = 1.0          # a factor on every sine and cosine (other encodings scale them)
+
     def __init__(self, head_dim: int, rotary_dim: int, theta: float, pairing: str = "half"):
         if pairing not in PAIRINGS:
             raise ValueError(f"unknown pairing {pairing!r}; known: {sorted(PAIRINGS)}")
@@ -57,6 +61,7 @@ class NoRotation(Part):
     graph_safe = True
     pairing_code = 0
     rotary_dim = 0
+    amplitude = 1.0
 
     def __init__(self):
         self._table = None
@@ -68,3 +73,35 @@ class NoRotation(Part):
 
     def prepare(self, device, act):
         self.table(device)
+
+
+@register_part("position", "yarn_rope")
+class YarnRotaryEncoding(RotaryEncoding):
+    """Rotary encoding whose slow pairs are stretched for sequences longer than the ``original`` length (YaRN).
+
+    With f_i = theta^(-2i / rotary_dim) and where(t) = rotary_dim ln(original / (2 pi t)) / (2 ln theta), the (fractional)
+    pair that makes t turns over the original length: lo = max(floor(where(fast)), 0), hi = min(ceil(where(slow)),
+    rotary_dim - 1), ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1); pair i turns at
+    f_i / factor * ramp_i + f_i (1 - ramp_i), and every sine and cosine is multiplied by ``amplitude`` =
+    0.1 ln(factor) + 1.  The table is worked out in double precision and rounded once; a mixer multiplies positions by
+    it in float32 and asks for ``amplitude`` beside ``table``, ``pairing_code`` and ``rotary_dim``."""
+
+    def __init__(self, head_dim: int, rotary_dim: int, theta: float, factor: float, original: float, fast: float,
+                 slow: float, pairing: str = "half"):
+        super().__init__(head_dim, rotary_dim, theta, pairing)
+        if not (factor >= 1.0 and original > 0 and fast > 0 and slow > 0 and theta > 1.0):
+            raise ValueError("YaRN needs factor >= 1, theta > 1 and positive original, fast and slow")
+        self.factor, self.original, self.fast, self.slow = float(factor), float(original), float(fast), float(slow)
+        self.amplitude = 0.1 * math.log(self.factor) + 1.0
+
+    def _where(self, turns: float) -> float:
+        return self.rotary_dim * math.log(self.original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
+
+    def frequencies(self) -> np.ndarray:
+        n = self.rotary_dim // 2
+        i = np.arange(n, dtype=np.float64)
+        f = np.power(float(self.theta), -2.0 * i / max(self.rotary_dim, 1))
+        lo = max(math.floor(self._where(self.fast)), 0)
+        hi = min(math.ceil(self._where(self.slow)), self.rotary_dim - 1)
+        ramp = np.clip((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        return (f / self.factor * ramp + f * (1.0 - ramp)).astype(np.float32)
