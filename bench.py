@@ -21,6 +21,13 @@ kernel by kernel.  The default run and its line are not touched by it.
 does the same for the Taminex design (a norm on every part's output only; attention with head norms, partial rotation
 and a sink; the delta rule with a decay per head; attention over a latent per position, shared between layers; a
 feed-forward of two matrices with squared relu) beside Qwen2-MoE with dense feed-forwards of as many weights.
+
+    python bench.py --design beronex [--design-sizes small,medium] [--layers 8]
+
+does it for the Beronex design (norms around every part; attention over a latent with a rotated key part and a latent for
+the queries; lightning attention; windowed attention with head norms behind a YaRN rotation, a gate per head and layers on
+another layer's keys and values; dense gated feed-forwards and clamped experts in turn) beside Qwen2-MoE with dense
+feed-forwards and experts in turn.
 """
 from __future__ import annotations
 
@@ -304,6 +311,38 @@ def qwen_dense_config_like(z: dict, layers: int, max_positions: int) -> dict:
                 mlp_only_layers=list(range(layers)), max_window_layers=layers, max_position_embeddings=max_positions)
 
 
+def beronex_config(z: dict, layers: int, max_positions: int) -> dict:
+    """`layers` layers in the order latent attention (queries through a latent, a rotated key part), lightning attention,
+    attention with a window, attention on that layer's keys and values; dense gated feed-forwards and routed experts in
+    turn.  The cached row of a latent layer is the latent and the rotated part, 512 numbers at most."""
+    H, G, D = z["heads"], z["kv_heads"], z["dim"]
+    dense = {"kind": "dense", "ff": z["dense_ff"]}
+    moe = {"kind": "moe", "router": {"experts": z["experts"], "top": z["top"]}, "expert": {"ff": z["ff"], "limit": 7.0}}
+    yarn = {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+    rank = min(z["kv_rank"], 512 - D // 2)
+    kinds = [
+        ("latent_attention", {"heads": H, "dim": D, "rot_dim": D // 2, "vdim": D, "kv_rank": rank, "q_rank": 3 * z["kv_rank"] // 2,
+                              "scale": (D + D // 2) ** -0.5, "rot": {"dims": D // 2, "base": 1e4, "scaling": yarn}}, dense),
+        ("lightning", {"heads": H, "dim": D, "vdim": D, "decay": [1.0 - 2.0 ** (-5.0 - 4.0 * h / H) for h in range(H)]}, moe),
+        ("attention", {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "mask": {"size": 1024},
+                       "rot": {"dims": D, "base": 1e6, "scaling": yarn}}, dense),
+        ("attention", {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "mask": {"size": 1024},
+                       "rot": {"dims": D, "base": 1e6, "scaling": yarn}}, moe),
+    ]
+    out = []
+    for i in range(layers):
+        kind, mixer, mlp = kinds[i % 4]
+        out.append({"type": kind, "mixer": dict(mixer, kv_from=i - 1) if i % 4 == 3 else dict(mixer), "mlp": mlp})
+    return {"architecture": "Beronex", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-5},
+            "embedding": {"scale": 1.0}, "layers": out}
+
+
+def qwen_mixed_config_like(z: dict, layers: int, max_positions: int) -> dict:
+    """Qwen2-MoE's layers with the dense gated feed-forward in every other layer and routed experts in the rest."""
+    return dict(qwen_config_like(z, layers, max_positions), intermediate_size=z["dense_ff"],
+                mlp_only_layers=list(range(0, layers, 2)))
+
+
 def qwen_config_like(z: dict, layers: int, max_positions: int) -> dict:
     return dict(A27B, vocab_size=z["vocab"], hidden_size=z["width"], num_hidden_layers=layers, num_attention_heads=z["heads"],
                 num_key_value_heads=z["kv_heads"], head_dim=z["dim"], moe_intermediate_size=z["ff"],
@@ -318,10 +357,11 @@ def design_comparison(args) -> int:
     from turboquant_cpp_amd.engine.step import Engine
     act, dev = args.dtype, "cuda:0"
     short = "bf16" if act == "bfloat16" else "fp32"
-    layers = args.layers or (8 if args.design == "taminex" else 6)
+    layers = args.layers or (6 if args.design == "felepel" else 8)
     context, prompts_at, batches = 2048, (512, 2048), (1, 8)
     design = {"felepel": ("Felepel", felepel_config, qwen_config_like),
-              "taminex": ("Taminex", taminex_config, qwen_dense_config_like)}[args.design]
+              "taminex": ("Taminex", taminex_config, qwen_dense_config_like),
+              "beronex": ("Beronex", beronex_config, qwen_mixed_config_like)}[args.design]
     out = {"metric": f"{design[0]} beside Qwen2-MoE at equal sizes: prompt and decode tok/s, and milliseconds by kernel",
            "unit": "tok/s", "dtype": short, "layer_runs": layers, "data": "synthetic", "sizes": {}}
 
@@ -425,7 +465,7 @@ def main() -> int:
     ap.add_argument("--seed", type=int, default=None)
     ap.add_argument("--no-workloads", action="store_true",
                     help="leave out the two workloads of unequal prompts that the default run adds under \"workloads\"")
-    ap.add_argument("--design", default=None, choices=["felepel", "taminex"],
+    ap.add_argument("--design", default=None, choices=["felepel", "taminex", "beronex"],
                     help="time this design beside Qwen2-MoE at equal sizes instead of the default workload")
     ap.add_argument("--design-sizes", default="small,medium", help="of " + ", ".join(DESIGN_SIZES))
     args = ap.parse_args()

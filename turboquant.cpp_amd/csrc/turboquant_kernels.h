@@ -41,6 +41,16 @@ int tq_rope_kv_write(const float* qkv, const void* bias, int bias_type, const in
         int rot, void* q_out, void* k_pool, void* v_pool, int page_size, int64_t page_stride, int T, int nh, int nkv,
         int hd, int write_kv, const int* cu_seqlens, const int* slots, const int* start, int B, int max_new,
         hipStream_t st);
+int tq_rope_kv_write_ex(const float* qkv, int64_t ld, const void* bias, int bias_type, const int* positions,
+        const int* seq_of_token, const int* block_table, int bt_stride, const float* inv_freq, int pairing, int rot,
+        float amp, float norm_eps, int norm_dim, void* q_out, void* k_pool, void* v_pool, int page_size,
+        int64_t page_stride, int T, int nh, int nkv, int hd, int write_kv, const int* cu_seqlens, const int* slots,
+        const int* start, int B, int max_new, hipStream_t st);
+int tq_gate_heads(const void* o, const float* gate, int64_t ldg, void* out, int M, int heads, int hd, int kind,
+        hipStream_t st);
+int tq_lead_norm(const float* in, int64_t ld_in, const void* w, int wtype, float eps, void* out, int out_is_act,
+        int64_t ld_out, int copies, int R, int lead, int Rp, int T, hipStream_t st);
+int tq_set_pair_limit(float limit);
 int tq_moe_combine(const float* y, const int* pair_slot, const float* weights, int topk, const float* shared,
         int S, int64_t shared_stride, const float* gate, float* out, int T, int H, hipStream_t st);
 int tq_embed_pos(const int* tokens, const int* positions, const void* table, const void* pos_table, int wtype, float* x,
@@ -130,6 +140,11 @@ int tq_delta_decode_h(const float* qn, const float* kn, const float* vc, const f
         const float* dt_bias, const float* norm_w, float eps, const float* P, int gate_kind, const int* cu_seqlens,
         const int* slots, float* state, int64_t state_stride, int H, int G, int D, int V, int taps, int B, void* out,
         hipStream_t st);
+// lightning.hip: linear attention with a constant decay per head (both libraries)
+int tq_lightning_scan(const float* P, int64_t ldp, const float* decay, const int* cu_seqlens, const int* slots,
+        float* state, int64_t state_stride, int B, int H, int D, int V, float* o, hipStream_t st);
+int tq_lightning_out(const float* o, const float* gate, int64_t ldg, const void* w, int wtype, float eps, void* out,
+        int T, int N, hipStream_t st);
 // head_gemm.hip: a product per head, out[t][h N + n] = sum_k a[t][h K + k] w[h][n][k] (both libraries)
 int tq_head_gemm(const void* a, int a_type, int64_t lda, const void* w, int wtype, void* out, int out_act, int64_t ldc,
         const float* gate, int64_t ldg, int gate_kind, int T, int H, int N, int K, hipStream_t st);
@@ -146,6 +161,13 @@ int tq_router_topk_grouped(const float* x, const void* wr, const void* shared_w,
 int tq_route_grouped(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk, int renorm,
         int groups, int keep, int* ids, float* weights, float* shared_gate, float* logits, int unit, int cap,
         int* sorted_token, int* pair_slot, int* tile_expert, int* n_tiles, int T, int H, hipStream_t st);
+int tq_router_topk_biased(const float* x, const void* wr, const void* shared_w, const float* bias, int wtype, int E,
+        int topk, int renorm, int groups, int keep, int* ids, float* weights, float* shared_gate, float* logits, int T,
+        int H, hipStream_t st);
+int tq_route_biased(const float* x, const void* wr, const void* shared_w, const float* bias, int wtype, int E,
+        int topk, int renorm, int groups, int keep, int* ids, float* weights, float* shared_gate, float* logits,
+        int unit, int cap, int* sorted_token, int* pair_slot, int* tile_expert, int* n_tiles, int T, int H,
+        hipStream_t st);
 // sampling.hip: greedy choice, negative log-likelihood, repetition penalty, temperature and top-p (both libraries; the two *_static entry points are declared in no_alloc.h)
 int tq_argmax(const float* logits, int R, int V, int* out, hipStream_t st);
 int tq_nll(const float* logits, int R, int V, const int* target, float* out, hipStream_t st);
