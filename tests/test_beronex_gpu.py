@@ -507,6 +507,41 @@ def test_lightning_kernels_with_a_state_carried_over(made):
         assert float(state[[0, 1, 3, 4, 6, 7]].abs().max()) == 0.0
 
 
+def test_lightning_in_chunks_on_the_matrix_cores(made):
+    """The chunked form of the recurrence: runs of one token, of a chunk less one, of a chunk, of a chunk and one, of
+    several chunks, side by side in slots in no order; a second step goes on from the states that the first one left."""
+    from turboquant_cpp_amd.csrc import ops
+    for case, layer in (("lightning_only", 0), ("odd", 0), ("ragged", 1), ("ragged", 2), ("wide", 0), ("wide", 3)):
+        _, cfg, w = made(case)
+        m, p = cfg["layers"][layer]["mixer"], f"l{layer}.mix."
+        H, D, V = m["heads"], m["dim"], m["vdim"]
+        rng = np.random.default_rng(10 + layer)
+        lens, slots = (200, 64, 1, 65, 130, 63), (6, 0, 3, 1, 5, 2)
+        hs = [rng.normal(size=(n + 70, cfg["width"])) for n in lens]
+        want = [plain.lightning(h, m, w, p, 1e-5, return_state=True) for h in hs]
+        w_in = np.concatenate([w[p + n] for n in ("q", "k", "v", "g")])
+        state = torch.zeros((8, H * D * V), dtype=torch.float32, device="cuda")
+        decay = f32(m["decay"])
+        outs = [[] for _ in lens]
+        for parts in ([h[:n] for h, n in zip(hs, lens)], [h[n:] for h, n in zip(hs, lens)]):
+            x = np.concatenate(parts)
+            cu = np.cumsum([0] + [len(q) for q in parts])
+            runs = {"cu_seqlens": torch.tensor(cu, dtype=torch.int32, device="cuda"),
+                    "slots": torch.tensor(slots, dtype=torch.int32, device="cuda"), "max_new": max(len(q) for q in parts)}
+            proj = f32(x @ w_in.T)
+            o = ops.lightning_chunked(proj, decay, runs, state, H, D, V, "float32")
+            out = ops.lightning_out(o, proj[:, 2 * H * D + H * V:], f32(w[p + "norm"]), 1e-5, "float32")
+            y = out.double().cpu().numpy() @ w[p + "o"].T
+            for i in range(len(lens)):
+                outs[i].append(y[cu[i]:cu[i + 1]])
+        for i in range(len(lens)):
+            got = np.concatenate(outs[i])
+            assert np.abs(got - want[i][0]).max() < 5e-5 * max(1.0, np.abs(want[i][0]).max()), (case, layer, i)
+            S = state[slots[i]].double().cpu().numpy().reshape(H, D, V)
+            assert np.abs(S - want[i][1]).max() < 5e-5 * max(1.0, np.abs(want[i][1]).max()), (case, layer, i)
+        assert float(state[[4, 7]].abs().max()) == 0.0
+
+
 def test_a_gate_per_head_and_a_norm_of_a_row_s_first_part():
     from turboquant_cpp_amd.csrc import ops
     rng = np.random.default_rng(1)

@@ -103,6 +103,8 @@ _SIGNATURES = {
                         _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     "tq_lightning_scan": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_ptr,
                           _c_ptr],
+    "tq_lightning_chunked": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int,
+                             _c_ptr, _c_int, _c_ptr, _c_ptr],
     "tq_lightning_out": [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_int, _c_f32, _c_ptr, _c_int, _c_int, _c_ptr],
 }
 # entry points that only one of the two libraries has
@@ -219,7 +221,7 @@ _KIND = {"gemm": "matmul", "gemm_mfma": "matmul", "gemm_f32": "matmul", "gemm_pa
          "router_topk": "moe", "route": "moe", "moe_align": "moe", "moe_combine": "moe",
          "delta_prep": "attn", "delta_scan": "attn", "delta_out": "attn", "delta_decode": "attn",
          "head_gemm": "matmul", "latent_norm": "attn", "gate_rows": "attn", "gate_heads": "attn",
-         "lightning_scan": "attn", "lightning_out": "attn"}
+         "lightning_scan": "attn", "lightning_chunked": "attn", "lightning_out": "attn"}
 
 
 def profile_begin() -> None:
@@ -1474,6 +1476,38 @@ def lightning_scan(proj: torch.Tensor, decay: torch.Tensor, runs: dict, state: t
     o = torch.empty((T, H * V), dtype=torch.float32, device=proj.device)
     _run(k, library(act).tq_lightning_scan(_ptr(proj), proj.stride(0), _ptr(decay), _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]),
                                            _ptr(state), state.stride(0), B, H, D, V, _ptr(o), _stream()))
+    return o
+
+
+LIGHTNING_CHUNK = 64           # tokens of a chunk of the chunked recurrence
+
+
+def lightning_chunked(proj: torch.Tensor, decay: torch.Tensor, runs: dict, state: torch.Tensor, num_heads: int, head_dim: int,
+                      value_dim: int, act) -> torch.Tensor:
+    """``lightning_scan`` for steps with long runs: the same function over chunks of 64 tokens on the matrix cores, in
+    float32 on both libraries (three launches: every chunk's own sum of k v^T, the states before the chunks, every
+    chunk's read-outs).  ``runs`` also names ``max_new``, the longest run.  Its sums are ordered by the chunks, which start
+    at the first token that the step brings: results agree with ``lightning_scan`` to rounding."""
+    k = "lightning_chunked"
+    H, D, V = num_heads, head_dim, value_dim
+    _need(isinstance(proj, torch.Tensor) and proj.is_cuda and proj.dtype == torch.float32 and proj.dim() == 2
+          and proj.stride(1) == 1 and proj.shape[1] >= 2 * H * D + 2 * H * V, k,
+          lambda: f"proj must be float32 [T, >= {2 * H * D + 2 * H * V}] on the GPU with unit stride along its rows")
+    _check(decay, k, "decay", torch.float32, (H,))
+    _check(state, k, "state", torch.float32)
+    _need(state.dim() == 2 and state.shape[1] == H * D * V, k, lambda: f"state must be [slots, {H * D * V}]")
+    _need(D <= 256, k, lambda: f"a key width of {D} is beyond the 256 this kernel takes")
+    B = runs["slots"].numel()
+    _check(runs["cu_seqlens"], k, "cu_seqlens", torch.int32, (B + 1,))
+    _check(runs["slots"], k, "slots", torch.int32, (B,))
+    T, max_new = proj.shape[0], int(runs["max_new"])
+    _need(1 <= max_new <= T, k, lambda: f"the longest run has {max_new} of {T} tokens")
+    chunks = T // LIGHTNING_CHUNK + B
+    scratch = torch.empty((chunks, H * D * V), dtype=torch.float32, device=proj.device)
+    o = torch.empty((T, H * V), dtype=torch.float32, device=proj.device)
+    _run(k, library(act).tq_lightning_chunked(_ptr(proj), proj.stride(0), _ptr(decay), _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]),
+                                              _ptr(state), state.stride(0), B, H, D, V, max_new, _ptr(scratch), chunks, _ptr(o),
+                                              _stream()))
     return o
 
 

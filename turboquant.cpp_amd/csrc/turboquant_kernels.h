@@ -143,6 +143,9 @@ int tq_delta_decode_h(const float* qn, const float* kn, const float* vc, const f
 // lightning.hip: linear attention with a constant decay per head (both libraries)
 int tq_lightning_scan(const float* P, int64_t ldp, const float* decay, const int* cu_seqlens, const int* slots,
         float* state, int64_t state_stride, int B, int H, int D, int V, float* o, hipStream_t st);
+int tq_lightning_chunked(const float* P, int64_t ldp, const float* decay, const int* cu_seqlens, const int* slots,
+        float* state, int64_t state_stride, int B, int H, int D, int V, int max_new, float* scratch, int scratch_chunks,
+        float* o, hipStream_t st);
 int tq_lightning_out(const float* o, const float* gate, int64_t ldg, const void* w, int wtype, float eps, void* out,
         int T, int N, hipStream_t st);
 // head_gemm.hip: a product per head, out[t][h N + n] = sum_k a[t][h K + k] w[h][n][k] (both libraries)

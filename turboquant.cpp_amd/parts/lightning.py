@@ -10,10 +10,12 @@ by sigmoid(W_g x) and go through the output product.  ``decay`` is a number per 
 
 The sequence's state is one row of float32 per slot (``StateNeed``): S as [heads, dim, vdim].  Activations of the
 projections, the recurrence, the norm and the gate are float32 on both libraries; the two products are the activation
-type's, the first one leaving its result in float32.  Four launches a step, prompt and decode alike: the product of all
+type's, the first one leaving its result in float32.  Four launches a decode step: the product of all
 projections (q | k | v | gate: one matrix), ``lightning_scan`` (the recurrence over each sequence's run of tokens, from
 and into the state of its slot, which the kernel finds through the slots on the device, so that a captured decode step
-replays for other slots), ``lightning_out`` (norm, weight, gate), the output product.
+replays for other slots), ``lightning_out`` (norm, weight, gate), the output product.  A step with a run of
+``chunked_from`` tokens or more takes ``lightning_chunked`` in the scan's place: the same sums over chunks of 64 tokens on
+the matrix cores in float32, every chunk's products side by side and only the states between chunks in order.
 """
 from __future__ import annotations
 
@@ -26,6 +28,7 @@ from .base import ParamSpec, Part, StateNeed, register_part
 @register_part("mixer", "lightning")
 class LightningAttention(Part):
     graph_safe = True       # what changes from step to step is read from the batch's device arrays only
+    chunked_from = 32       # a step whose longest run has this many tokens takes the chunked form
 
     def __init__(self, hidden_size: int, num_heads: int, head_dim: int, value_dim: int, decay, eps: float):
         decay = [float(d) for d in decay]
@@ -63,6 +66,10 @@ class LightningAttention(Part):
     def forward(self, normed, ctx, entry):
         H, D, V = self.num_heads, self.head_dim, self.value_dim
         proj = ops.gemm(normed, self.in_weight, ctx.act)                            # float32 [T, q | k | v | gate]
-        o = ops.lightning_scan(proj, self.decay, ctx.batch.runs(), ctx.state(entry), H, D, V, ctx.act)
+        runs = ctx.batch.runs()
+        if not runs["decode"] and runs["max_new"] >= self.chunked_from and not ctx.capturing:
+            o = ops.lightning_chunked(proj, self.decay, runs, ctx.state(entry), H, D, V, ctx.act)
+        else:
+            o = ops.lightning_scan(proj, self.decay, runs, ctx.state(entry), H, D, V, ctx.act)
         out = ops.lightning_out(o, proj[:, 2 * H * D + H * V:], self.out_norm, self.eps, ctx.act)
         return ops.gemm(out, self.out_weight, ctx.act, partial_sums=True)
