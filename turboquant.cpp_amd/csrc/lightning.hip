@@ -138,8 +138,47 @@ __device__ __forceinline__ int lc_chunk_base(const int* __restrict__ cu_seqlens,
   return base;
 }
 
+// A chunk's rows of one projection on their way into LDS: first every load (all in flight together), then the silu and
+// the stores.  W numbers a row (WP in LDS, a multiple of 16; zeros behind W and behind the chunk's nc tokens).  VEC: rows
+// start at multiples of 16 bytes and W is a multiple of four.
+template <int WP, bool VEC>
+struct LcRows {
+  static constexpr int N = VEC ? LC_T * WP / 4 / 256 : LC_T * WP / 256;
+  float x[VEC ? 4 * N : N];
+  __device__ __forceinline__ void fetch(const float* __restrict__ src, int64_t ld, int nc, int W, int tid) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int idx = tid + 256 * i;
+      if (VEC) {
+        const int s = idx / (WP / 4), d = 4 * (idx % (WP / 4));
+        const float4 v = s < nc && d < W ? *reinterpret_cast<const float4*>(src + (size_t)s * ld + d) : float4{0.f, 0.f, 0.f, 0.f};
+        x[4 * i] = v.x, x[4 * i + 1] = v.y, x[4 * i + 2] = v.z, x[4 * i + 3] = v.w;
+      } else {
+        const int s = idx / WP, d = idx % WP;
+        x[i] = s < nc && d < W ? src[(size_t)s * ld + d] : 0.f;
+      }
+    }
+  }
+  // dst[s * ld + d] = silu(x) * (wt ? wt[s] : 1)
+  __device__ __forceinline__ void store(float* __restrict__ dst, int ld, const float* __restrict__ wt, int tid) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int idx = tid + 256 * i;
+      if (VEC) {
+        const int s = idx / (WP / 4), d = 4 * (idx % (WP / 4));
+        const float w = wt ? wt[s] : 1.f;
+        *reinterpret_cast<float4*>(dst + s * ld + d) =
+            float4{w * ln_silu(x[4 * i]), w * ln_silu(x[4 * i + 1]), w * ln_silu(x[4 * i + 2]), w * ln_silu(x[4 * i + 3])};
+      } else {
+        const int s = idx / WP, d = idx % WP;
+        dst[s * ld + d] = (wt ? wt[s] : 1.f) * ln_silu(x[i]);
+      }
+    }
+  }
+};
+
 // grid (ceil(V / LC_V), H, B * NC), block 256: L_c [D][LC_V columns] = K^T (w . V), a wave to 16 value channels.
-template <int ND>
+template <int ND, bool VEC>
 __global__ __launch_bounds__(256) void lightning_chunk_state_kernel(const float* __restrict__ P, int64_t ldp,
                                                                     const float* __restrict__ decay,
                                                                     const int* __restrict__ cu_seqlens, int NC, int cap,
@@ -159,15 +198,13 @@ __global__ __launch_bounds__(256) void lightning_chunk_state_kernel(const float*
   if (tid < LC_T) wt[tid] = tid < nc ? powf(lam, (float)(nc - 1 - tid)) : 0.f;
   const float* k0 = P + (size_t)(t0 + c * LC_T) * ldp + (size_t)H * D + (size_t)h * D;
   const float* vv0 = P + (size_t)(t0 + c * LC_T) * ldp + (size_t)2 * H * D + (size_t)h * V + v0;
-  for (int idx = tid; idx < LC_T * DP; idx += 256) {
-    const int s = idx / DP, d = idx % DP;
-    ks[s * KLD + d] = s < nc && d < D ? ln_silu(k0[(size_t)s * ldp + d]) : 0.f;
-  }
+  LcRows<DP, VEC> kr_;
+  LcRows<LC_V, VEC> vr_;
+  kr_.fetch(k0, ldp, nc, D, tid);
+  vr_.fetch(vv0, ldp, nc, V - v0, tid);
+  kr_.store(ks, KLD, nullptr, tid);
   __syncthreads();
-  for (int idx = tid; idx < LC_T * LC_V; idx += 256) {
-    const int s = idx / LC_V, i = idx % LC_V;
-    vs[s * LC_VLD + i] = s < nc && v0 + i < V ? wt[s] * ln_silu(vv0[(size_t)s * ldp + i]) : 0.f;
-  }
+  vr_.store(vs, LC_VLD, wt, tid);
   __syncthreads();
   const int wave = tid / 64, lane = tid % 64, g = lane / 16, r = lane % 16;
   lc_f32x4 acc[ND];
@@ -219,7 +256,7 @@ __global__ __launch_bounds__(256) void lightning_chunk_prefix_kernel(const float
 }
 
 // grid (ceil(V / LC_V), H, B * NC), block 256: a chunk's read-outs for LC_V value channels, a wave to 16 tokens.
-template <int ND>
+template <int ND, bool VEC>
 __global__ __launch_bounds__(256) void lightning_chunk_out_kernel(const float* __restrict__ P, int64_t ldp,
                                                                   const float* __restrict__ decay,
                                                                   const int* __restrict__ cu_seqlens, int NC, int cap,
@@ -237,23 +274,32 @@ __global__ __launch_bounds__(256) void lightning_chunk_out_kernel(const float* _
   const int gi = lc_chunk_base(cu_seqlens, b) + c;
   if (gi >= cap) return;
   const int nc = min(LC_T, n - c * LC_T), tid = threadIdx.x;
+  const int wave = tid / 64, lane = tid % 64, g = lane / 16, r = lane % 16;
+  // the state before the chunk, as the last product's operand: asked for first, so that it arrives while the rest is staged
+  constexpr int AHEAD = DP / 4 > 32 ? 32 : DP / 4;
+  const float* sb = S + ((size_t)gi * H + h) * D * V + v0 + r;
+  float sv[AHEAD][4];
+#pragma unroll
+  for (int k4 = 0; k4 < AHEAD; ++k4)
+#pragma unroll
+    for (int cv = 0; cv < 4; ++cv)
+      sv[k4][cv] = 4 * k4 + g < D && v0 + 16 * cv + r < V ? sb[(size_t)(4 * k4 + g) * V + 16 * cv] : 0.f;
   const float lam = decay[h];
   if (tid <= LC_T) pw[tid] = powf(lam, (float)tid);
   const float* q0 = P + (size_t)(t0 + c * LC_T) * ldp + (size_t)h * D;
   const float* k0 = q0 + (size_t)H * D;
   const float* vv0 = P + (size_t)(t0 + c * LC_T) * ldp + (size_t)2 * H * D + (size_t)h * V + v0;
-  for (int idx = tid; idx < LC_T * DP; idx += 256) {
-    const int s = idx / DP, d = idx % DP;
-    const bool in = s < nc && d < D;
-    qs[s * QLD + d] = in ? ln_silu(q0[(size_t)s * ldp + d]) : 0.f;
-    ks[s * QLD + d] = in ? ln_silu(k0[(size_t)s * ldp + d]) : 0.f;
-  }
-  for (int idx = tid; idx < LC_T * LC_V; idx += 256) {
-    const int s = idx / LC_V, i = idx % LC_V;
-    vs[s * LC_VLD + i] = s < nc && v0 + i < V ? ln_silu(vv0[(size_t)s * ldp + i]) : 0.f;
+  {
+    LcRows<DP, VEC> qr_, kr_;
+    LcRows<LC_V, VEC> vr_;
+    qr_.fetch(q0, ldp, nc, D, tid);
+    kr_.fetch(k0, ldp, nc, D, tid);
+    vr_.fetch(vv0, ldp, nc, V - v0, tid);
+    qr_.store(qs, QLD, nullptr, tid);
+    kr_.store(ks, QLD, nullptr, tid);
+    vr_.store(vs, LC_VLD, nullptr, tid);
   }
   __syncthreads();
-  const int wave = tid / 64, lane = tid % 64, g = lane / 16, r = lane % 16;
   // scores of the wave's 16 tokens against the tokens of the column tiles up to its own
   lc_f32x4 sc[4];
 #pragma unroll
@@ -288,9 +334,14 @@ __global__ __launch_bounds__(256) void lightning_chunk_out_kernel(const float* _
     for (int cv = 0; cv < 4; ++cv) acc[cv] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, vr[16 * cv], acc[cv], 0, 0, 0);
   }
   // what the state before the chunk adds: q S, each row times decay^(t + 1)
-  const float* sb = S + ((size_t)gi * H + h) * D * V + v0 + r;
-#pragma unroll 4
-  for (int k4 = 0; k4 < DP / 4; ++k4) {
+#pragma unroll
+  for (int k4 = 0; k4 < AHEAD; ++k4) {
+    const float a = qrow[4 * k4];
+#pragma unroll
+    for (int cv = 0; cv < 4; ++cv) far[cv] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, sv[k4][cv], far[cv], 0, 0, 0);
+  }
+#pragma unroll 8
+  for (int k4 = AHEAD; k4 < DP / 4; ++k4) {
     const float a = qrow[4 * k4];
     const int d = 4 * k4 + g;
 #pragma unroll
@@ -310,7 +361,7 @@ __global__ __launch_bounds__(256) void lightning_chunk_out_kernel(const float* _
   }
 }
 
-template <int ND>
+template <int ND, bool VEC>
 static int lightning_chunked_launch(const float* P, int64_t ldp, const float* decay, const int* cu_seqlens, const int* slots,
                                     float* state, int64_t state_stride, int B, int NC, int cap, int H, int D, int V,
                                     float* scratch, float* o, hipStream_t st) {
@@ -318,16 +369,18 @@ static int lightning_chunked_launch(const float* P, int64_t ldp, const float* de
   const size_t sh_state = ((size_t)LC_T * KLD + (size_t)LC_T * LC_VLD + LC_T) * sizeof(float);
   const size_t sh_out = ((size_t)LC_T * QLD + (size_t)LC_T * KROWS + (size_t)LC_T * LC_VLD + LC_T + 4) * sizeof(float);
   if (sh_state > 48 * 1024)
-    (void)hipFuncSetAttribute((const void*)lightning_chunk_state_kernel<ND>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh_state);
+    (void)hipFuncSetAttribute((const void*)lightning_chunk_state_kernel<ND, VEC>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)sh_state);
   if (sh_out > 48 * 1024)
-    (void)hipFuncSetAttribute((const void*)lightning_chunk_out_kernel<ND>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh_out);
+    (void)hipFuncSetAttribute((const void*)lightning_chunk_out_kernel<ND, VEC>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)sh_out);
   const dim3 grid((V + LC_V - 1) / LC_V, H, B * NC);
-  hipLaunchKernelGGL(lightning_chunk_state_kernel<ND>, grid, dim3(256), sh_state, st, P, ldp, decay, cu_seqlens, NC, cap, H, D, V,
-                     scratch);
+  hipLaunchKernelGGL((lightning_chunk_state_kernel<ND, VEC>), grid, dim3(256), sh_state, st, P, ldp, decay, cu_seqlens, NC, cap, H,
+                     D, V, scratch);
   hipLaunchKernelGGL(lightning_chunk_prefix_kernel, dim3((D * V + 255) / 256, H, B), dim3(256), 0, st, decay, cu_seqlens, slots,
                      state, state_stride, cap, H, D, V, scratch);
-  hipLaunchKernelGGL(lightning_chunk_out_kernel<ND>, grid, dim3(256), sh_out, st, P, ldp, decay, cu_seqlens, NC, cap, H, D, V,
-                     scratch, o);
+  hipLaunchKernelGGL((lightning_chunk_out_kernel<ND, VEC>), grid, dim3(256), sh_out, st, P, ldp, decay, cu_seqlens, NC, cap, H, D,
+                     V, scratch, o);
   TQ_LAUNCH_CHECK();
   return 0;
 }
@@ -343,8 +396,13 @@ TQ_API int tq_lightning_chunked(const float* P, int64_t ldp, const float* decay,
     return TQ_ERR_BAD_ARG;
   const int NC = (max_new + LC_T - 1) / LC_T;
   if (D > 256 || H > 65535 || (int64_t)B * NC > 65535 || (int64_t)D * V > (int64_t)256 * 65535) return TQ_ERR_UNSUPPORTED;
-#define TQ_LC(NDV) \
-  return lightning_chunked_launch<NDV>(P, ldp, decay, cu_seqlens, slots, state, state_stride, B, NC, scratch_chunks, H, D, V, scratch, o, st)
+  // whole rows of four floats: every row of every head starts at a multiple of 16 bytes
+  const bool vec = D % 4 == 0 && V % 4 == 0 && ldp % 4 == 0 && (uintptr_t)P % 16 == 0;
+#define TQ_LC(NDV)                                                                                                        \
+  return vec ? lightning_chunked_launch<NDV, true>(P, ldp, decay, cu_seqlens, slots, state, state_stride, B, NC,          \
+                                                   scratch_chunks, H, D, V, scratch, o, st)                               \
+             : lightning_chunked_launch<NDV, false>(P, ldp, decay, cu_seqlens, slots, state, state_stride, B, NC,         \
+                                                    scratch_chunks, H, D, V, scratch, o, st)
   if (D <= 16) TQ_LC(1);
   if (D <= 32) TQ_LC(2);
   if (D <= 64) TQ_LC(4);
