@@ -430,13 +430,16 @@ __device__ __forceinline__ void load_query(bf16x8 (&qf)[(DT + 1) / 2], const bf1
 // the other, and the tile after that is on its way from memory into registers meanwhile: one barrier per tile.
 #define KPAD 8
 #define VSTR 72
+#ifndef ATTN_TWO_BUFFERS_UP_TO
+#define ATTN_TWO_BUFFERS_UP_TO 8      // heads of up to 16 times this many numbers keep two tiles in LDS
+#endif
 
 // Heads wider than 256 (DT = 32; an attention over compressed rows that all heads share has such): one buffer instead of
 // two, since two tiles of 64 x 512 keys and values are beyond the LDS, and a wave to a SIMD, since a column's sums
 // alone are 128 registers; the next tile still travels from memory into registers while this one is worked on.
 template <int DT, int QG, bool EXACT, bool MOD>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DT > 16 ? 1 : 2))) void attn_prefill_kernel(AttnArgs a, int n_blocks, int B) {
-  constexpr bool ONEBUF = DT > 16;
+  constexpr bool ONEBUF = DT > ATTN_TWO_BUFFERS_UP_TO;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   constexpr int QW = 16 * QG;
   constexpr int KCH = (TILE * 2 * DT + 255) / 256;      // 16-byte chunks of a key tile per thread
@@ -713,7 +716,7 @@ __global__ __launch_bounds__(256) void attn_join_kernel(AttnArgs a) {
 // ------------------------------------------------------------------------------------------ launch
 template <int DT, int QG, bool EXACT, bool MOD>
 static int launch_prefill_as(const AttnArgs& a, int B, int max_new, hipStream_t st) {
-  const size_t shmem = (DT > 16 ? 1 : 2) * (EXACT ? (size_t)2 * TILE * a.hd : (size_t)TILE * (a.hd + KPAD) + (size_t)a.hd * VSTR) * sizeof(bf16_t);
+  const size_t shmem = (DT > ATTN_TWO_BUFFERS_UP_TO ? 1 : 2) * (EXACT ? (size_t)2 * TILE * a.hd : (size_t)TILE * (a.hd + KPAD) + (size_t)a.hd * VSTR) * sizeof(bf16_t);
   if (shmem > 48 * 1024)
     (void)hipFuncSetAttribute((const void*)attn_prefill_kernel<DT, QG, EXACT, MOD>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   const int n_blocks = (max_new + 64 * QG - 1) / (64 * QG);
