@@ -1198,6 +1198,8 @@ def test_sample_topp_distribution(ops):
 @pytest.mark.parametrize("nh,nkv,hd,window,page", [(4, 4, 16, None, 64), (6, 2, 48, 24, 64), (3, 1, 80, 70, 128),
                                                      (16, 16, 128, None, 64), (40, 2, 32, 200, 64), (2, 1, 256, None, 64),
                                                      (5, 5, 96, 1, 64), (8, 2, 64, 100, 64),
+                                                     # a head of 192 has a kernel of its own
+                                                     (4, 2, 192, None, 64), (3, 3, 192, 100, 128),
                                                      # enough heads for two token groups per wave
                                                      (48, 6, 128, None, 64), (48, 4, 64, 100, 64), (44, 4, 48, 30, 64),
                                                      # head sizes that are a multiple of 4 only (the 32-bit kernels take them)
@@ -1207,6 +1209,18 @@ def test_attention_tiled(ops, act, nh, nkv, hd, window, page):
     """The matrix-core kernels of both types (whole runs of tokens, and one token per sequence split over the cache)
     against the plain attention: unequal lengths, a sequence that goes on from a cached prefix, groups of more than
     16 heads."""
+    attention_tiled(ops, act, nh, nkv, hd, window, page)
+
+
+@pytest.mark.parametrize("nh,nkv,hd,width,window", [(4, 4, 192, 128, None), (48, 48, 192, 128, None), (5, 1, 192, 64, 90),
+                                                     (3, 3, 192, 192, None), (4, 2, 128, 64, None), (2, 2, 80, 48, 70)])
+def test_attention_with_keys_wider_than_values(ops, nh, nkv, hd, width, window):
+    """Values that are zeros behind their first ``width`` numbers, and the call says so: the result is the plain
+    attention's (zeros there), whether or not the kernel that runs leaves those dimensions out."""
+    attention_tiled(ops, "bfloat16", nh, nkv, hd, window, 64, value_width=width)
+
+
+def attention_tiled(ops, act, nh, nkv, hd, window, page, value_width=None):
     lens = [1, 19, 150, 333]
     layers, layer = 3, 1
     table, slots, page_stride, kp, vp = paged_setup(lens, page, nkv, hd, layers, act, 130)
@@ -1217,6 +1231,8 @@ def test_attention_tiled(ops, act, nh, nkv, hd, window, page):
         qs.append(rnd((n, nh, hd), adt(act), 131 + i))
         ks.append(rnd((n, nkv, hd), adt(act), 135 + i))
         vs.append(rnd((n, nkv, hd), adt(act), 139 + i))
+        if value_width is not None:
+            vs[-1][:, :, value_width:] = 0
         for p in range(n):
             for h in range(nkv):
                 base = int(table[slots[i], p // page]) * page_stride + off + (h * page + p % page) * hd
@@ -1225,6 +1241,7 @@ def test_attention_tiled(ops, act, nh, nkv, hd, window, page):
                 vp[vbase:vbase + hd * page:page] = vs[i][p, h]
     kd, vd, td = kp.to(DEV), vp.to(DEV), table.to(DEV)
     ref = [ref_attention(a, b, c, window, scale).reshape(-1, nh * hd) for a, b, c in zip(qs, ks, vs)]
+    more = {} if value_width is None else {"value_width": value_width}
 
     def run(first):          # tokens first[i] .. lens[i]-1 of every sequence in one call
         new = [n - f for n, f in zip(lens, first)]
@@ -1237,7 +1254,7 @@ def test_attention_tiled(ops, act, nh, nkv, hd, window, page):
                 "start": torch.tensor([first[i] for i in keep], dtype=torch.int32).to(DEV),
                 "max_new": max(new), "max_end": max(lens[i] for i in keep), "decode": all(new[i] == 1 for i in keep)}
         out = ops.attention(q.to(DEV), kd, vd, off, positions.to(DEV), slot_of.to(DEV), td, page, page_stride, nh, nkv,
-                            hd, window, scale, act, runs=runs).cpu()
+                            hd, window, scale, act, runs=runs, **more).cpu()
         want = torch.cat([ref[i][first[i]:] for i in keep])
         return (out.double() - want).abs().max().item()
 

@@ -134,7 +134,9 @@ __device__ __forceinline__ float group_sum(float v) {
 // and compute unit, rows padded by 16 bytes at about 120.
 template <int DT>
 __device__ __forceinline__ int k_swz(int row, int ch) {
-  const int g = DT == 4 ? (((row >> 1) & 1) | (((row >> 3) & 3) << 1)) : ((row & 3) | (((row >> 3) & 3) << 2));
+  // (rows whose number of chunks is no power of two, a head of 192: the lowest three bits of ch only, which stays in the row)
+  const int g = DT == 4 ? (((row >> 1) & 1) | (((row >> 3) & 3) << 1))
+              : (2 * DT) & (2 * DT - 1) ? ((row & 3) | (((row >> 3) & 1) << 2)) : ((row & 3) | (((row >> 3) & 3) << 2));
   return row * (16 * DT) + ((ch ^ g) << 3);
 }
 __device__ __forceinline__ int v_swz(int d, int ch) { return d * TILE + ((ch ^ (d & 7)) << 3); }
@@ -437,17 +439,20 @@ __device__ __forceinline__ void load_query(bf16x8 (&qf)[(DT + 1) / 2], const bf1
 // Heads wider than 256 (DT = 32; an attention over compressed rows that all heads share has such): one buffer instead of
 // two, since two tiles of 64 x 512 keys and values are beyond the LDS, and a wave to a SIMD, since a column's sums
 // alone are 128 registers; the next tile still travels from memory into registers while this one is worked on.
-template <int DT, int QG, bool EXACT, bool MOD>
+// VD < DT: the values' first 16 VD dimensions alone are summed and written (zeros behind them up to hd): an attention
+// whose keys are wider than its values, laid out at the keys' width.
+template <int DT, int QG, bool EXACT, bool MOD, int VD = DT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DT > 16 ? 1 : 2))) void attn_prefill_kernel(AttnArgs a, int n_blocks, int B) {
   constexpr bool ONEBUF = DT > ATTN_TWO_BUFFERS_UP_TO;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   constexpr int QW = 16 * QG;
   constexpr int KCH = (TILE * 2 * DT + 255) / 256;      // 16-byte chunks of a key tile per thread
-  constexpr int VCH = (16 * DT * 8 + 255) / 256;        // and of a value tile
+  constexpr int VCH = (16 * VD * 8 + 255) / 256;        // and of a value tile
+  static_assert(VD <= DT && (VD == DT || EXACT), "fewer value dimensions than key dimensions: for exact head sizes");
   const int hd = EXACT ? 16 * DT : a.hd, kcpr = hd / 8;
   // elements of one buffer: keys [TILE][hd + KPAD], values [hd][VSTR]; swizzled instead of padded when EXACT
   const int kstr = EXACT ? hd : hd + KPAD, vstr = EXACT ? TILE : VSTR;
-  const int buf = TILE * kstr + hd * vstr;
+  const int buf = TILE * kstr + (VD < DT ? 16 * VD : hd) * vstr;
   bf16_t* Ks = (bf16_t*)smem_raw;
   bf16_t* Vs = Ks + TILE * kstr;
   const int per_block = a.nh * B;
@@ -464,7 +469,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DT > 16 ? 1
 
   int p_q[QG], lo_q[QG];
   bf16x8 qf[QG][(DT + 1) / 2];
-  f32x4 o[QG][DT];
+  f32x4 o[QG][VD];
   float m_run[QG], l_run[QG];
 #pragma unroll
   for (int g = 0; g < QG; ++g) {
@@ -474,7 +479,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DT > 16 ? 1
     lo_q[g] = reach_lo(p_q[g], a.window, a.mod.chunk);
     load_query<DT>(qf[g], a.q + ((size_t)(t0 + (valid ? qi : 0)) * a.nh + h) * hd, hd, valid);
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) o[g][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int dt = 0; dt < VD; ++dt) o[g][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     m_run[g] = -INFINITY;
     l_run[g] = 0.f;
     if (a.mod.sink) {       // a score without key or value, counted once; maxima are in units of log2
@@ -507,7 +512,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DT > 16 ? 1
     in_lds = EXACT ? k_swz<DT>(row, ch) : row * kstr + ch * 8;
   };
   auto v_place = [&](int j, int& in_mem, int& in_lds) {
-    const int i = min(tid + j * 256, hd * 8 - 1), d = i / 8, ch = i % 8;
+    const int i = min(tid + j * 256, (VD < DT ? 16 * VD : hd) * 8 - 1), d = i / 8, ch = i % 8;
     in_mem = d * a.page_size + ch * 8;
     in_lds = EXACT ? v_swz(d, ch) : d * vstr + ch * 8;
   };
@@ -549,7 +554,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DT > 16 ? 1
       if (tile >= wave_beg && tile < wave_end) {
         const int pos0 = tile * TILE;
         const bool masked = pos0 + TILE - 1 > wave_first || pos0 < wave_lo_last;
-        tile_step<DT, QG, EXACT, EXACT, false, MOD>(o, m_run, l_run, qf, Ks, kstr, Vs, vstr, hd, pos0, p_q, lo_q,
+        tile_step<DT, QG, EXACT, EXACT, false, MOD, VD>(o, m_run, l_run, qf, Ks, kstr, Vs, vstr, hd, pos0, p_q, lo_q,
                                         a.scale * LOG2E, masked, cm);
       }
       __syncthreads();
@@ -567,7 +572,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DT > 16 ? 1
     if (tile >= wave_beg && tile < wave_end) {
       const int pos0 = tile * TILE;
       const bool masked = pos0 + TILE - 1 > wave_first || pos0 < wave_lo_last;
-      tile_step<DT, QG, EXACT, EXACT, false, MOD>(o, m_run, l_run, qf, Ks + cur, kstr, Vs + cur, vstr, hd, pos0, p_q, lo_q,
+      tile_step<DT, QG, EXACT, EXACT, false, MOD, VD>(o, m_run, l_run, qf, Ks + cur, kstr, Vs + cur, vstr, hd, pos0, p_q, lo_q,
                                       a.scale * LOG2E, masked, cm);
     }
     __syncthreads();
@@ -581,12 +586,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DT > 16 ? 1
     const float inv = 1.0f / l_run[g];
     bf16_t* orow = a.out + ((size_t)(t0 + p_q[g] - start) * a.nh + h) * hd;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
+    for (int dt = 0; dt < VD; ++dt) {
       if (16 * dt < hd) {
         const u32x2 w = {pack2(o[g][dt][0] * inv, o[g][dt][1] * inv), pack2(o[g][dt][2] * inv, o[g][dt][3] * inv)};
         *reinterpret_cast<u32x2*>(orow + 16 * dt + 4 * c) = w;
       }
     }
+#pragma unroll
+    for (int dt = VD; dt < DT; ++dt) *reinterpret_cast<u32x2*>(orow + 16 * dt + 4 * c) = u32x2{0u, 0u};
   }
 }
 
@@ -714,21 +721,21 @@ __global__ __launch_bounds__(256) void attn_join_kernel(AttnArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------ launch
-template <int DT, int QG, bool EXACT, bool MOD>
+template <int DT, int QG, bool EXACT, bool MOD, int VD = DT>
 static int launch_prefill_as(const AttnArgs& a, int B, int max_new, hipStream_t st) {
-  const size_t shmem = (DT > ATTN_TWO_BUFFERS_UP_TO ? 1 : 2) * (EXACT ? (size_t)2 * TILE * a.hd : (size_t)TILE * (a.hd + KPAD) + (size_t)a.hd * VSTR) * sizeof(bf16_t);
+  const size_t shmem = (DT > ATTN_TWO_BUFFERS_UP_TO ? 1 : 2) * (EXACT ? (size_t)TILE * (a.hd + 16 * VD) : (size_t)TILE * (a.hd + KPAD) + (size_t)a.hd * VSTR) * sizeof(bf16_t);
   if (shmem > 48 * 1024)
-    (void)hipFuncSetAttribute((const void*)attn_prefill_kernel<DT, QG, EXACT, MOD>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    (void)hipFuncSetAttribute((const void*)attn_prefill_kernel<DT, QG, EXACT, MOD, VD>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   const int n_blocks = (max_new + 64 * QG - 1) / (64 * QG);
   if ((int64_t)n_blocks * a.nh * B > 0x7fffffff) return TQ_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL((attn_prefill_kernel<DT, QG, EXACT, MOD>), dim3(n_blocks * a.nh * B), dim3(256), shmem, st, a, n_blocks, B);
+  hipLaunchKernelGGL((attn_prefill_kernel<DT, QG, EXACT, MOD, VD>), dim3(n_blocks * a.nh * B), dim3(256), shmem, st, a, n_blocks, B);
   return 0;
 }
 // (the kernels that cap or bias scores are instantiations of their own, so that the others carry nothing of it)
-template <int DT, int QG, bool EXACT>
+template <int DT, int QG, bool EXACT, int VD = DT>
 static int launch_prefill(const AttnArgs& a, int B, int max_new, hipStream_t st) {
-  return (a.mod.cap > 0.f || a.mod.r1) ? launch_prefill_as<DT, QG, EXACT, true>(a, B, max_new, st)
-                                       : launch_prefill_as<DT, QG, EXACT, false>(a, B, max_new, st);
+  return (a.mod.cap > 0.f || a.mod.r1) ? launch_prefill_as<DT, QG, EXACT, true, VD>(a, B, max_new, st)
+                                       : launch_prefill_as<DT, QG, EXACT, false, VD>(a, B, max_new, st);
 }
 template <int DT, bool EXACT, bool MOD>
 static void launch_decode_as(const AttnArgs& a, int B, int grid_runs, hipStream_t st) {
@@ -761,13 +768,16 @@ TQ_API int64_t tq_attention_decode_scratch(int B, int nh, int hd, int max_end) {
 // decode != 0: every sequence brings exactly one token.  max_new: longest run of new tokens of a sequence;
 // max_end: largest position + 1 that any token of the step has.
 // softcap, r1, r2, chunk, sink: see score_mod.h (0, null, null, 0, null: nothing).
-TQ_API int tq_attention_mfma_mod(const void* q, const void* k_pool, const void* v_pool, const int* block_table,
-                                 int bt_stride, const int* cu_seqlens, const int* slots, const int* start, int page_size,
-                                 int64_t page_stride, int B, int nh, int nkv, int hd, int window, float scale,
-                                 float softcap, const float* r1, const float* r2, int chunk, const float* sink,
-                                 void* out, float* partial, int decode, int max_new, int max_end, hipStream_t st) {
+// value_width (0: hd): the values' first numbers that matter; a head's value rows behind them are zeros, and so is the
+// output there, which lets a kernel leave them out.
+TQ_API int tq_attention_mfma_wide_keys(const void* q, const void* k_pool, const void* v_pool, const int* block_table,
+                                       int bt_stride, const int* cu_seqlens, const int* slots, const int* start, int page_size,
+                                       int64_t page_stride, int B, int nh, int nkv, int hd, int window, float scale,
+                                       float softcap, const float* r1, const float* r2, int chunk, const float* sink,
+                                       void* out, float* partial, int decode, int max_new, int max_end, int value_width,
+                                       hipStream_t st) {
   if (B <= 0) return 0;
-  if ((r1 == nullptr) != (r2 == nullptr) || chunk < 0 || softcap < 0.f) return TQ_ERR_BAD_ARG;
+  if ((r1 == nullptr) != (r2 == nullptr) || chunk < 0 || softcap < 0.f || value_width < 0 || value_width > hd) return TQ_ERR_BAD_ARG;
   if (hd % 16 != 0 || hd < 16 || hd > 512 || page_size % TILE != 0 || nkv <= 0 || nh % nkv != 0)
     return TQ_ERR_UNSUPPORTED;
   if (nh > 65535 || B > 65535 || page_stride % 8 != 0 || !(scale > 0.f)) return TQ_ERR_UNSUPPORTED;
@@ -796,6 +806,10 @@ TQ_API int tq_attention_mfma_mod(const void* q, const void* k_pool, const void* 
     if (dt == 4) rc = two ? launch_prefill<4, 2, true>(a, B, max_new, st) : launch_prefill<4, 1, true>(a, B, max_new, st);
     else if (dt == 8) rc = two ? launch_prefill<8, 2, true>(a, B, max_new, st) : launch_prefill<8, 1, true>(a, B, max_new, st);
     else if (dt == 16) rc = launch_prefill<16, 1, true>(a, B, max_new, st);
+    // a head of 192 (128 plain and 64 rotated numbers of a latent attention's keys), with values of 128 or of 192
+    else if (dt == 12 && value_width > 0 && value_width <= 128)
+      rc = two ? launch_prefill<12, 2, true, 8>(a, B, max_new, st) : launch_prefill<12, 1, true, 8>(a, B, max_new, st);
+    else if (dt == 12) rc = launch_prefill<12, 1, true>(a, B, max_new, st);
     else if (dt < 4) rc = two ? launch_prefill<4, 2, false>(a, B, max_new, st) : launch_prefill<4, 1, false>(a, B, max_new, st);
     else if (dt < 8) rc = two ? launch_prefill<8, 2, false>(a, B, max_new, st) : launch_prefill<8, 1, false>(a, B, max_new, st);
     else if (dt < 16) rc = launch_prefill<16, 1, false>(a, B, max_new, st);
@@ -805,6 +819,16 @@ TQ_API int tq_attention_mfma_mod(const void* q, const void* k_pool, const void* 
   }
   TQ_LAUNCH_CHECK();
   return 0;
+}
+
+TQ_API int tq_attention_mfma_mod(const void* q, const void* k_pool, const void* v_pool, const int* block_table,
+                                 int bt_stride, const int* cu_seqlens, const int* slots, const int* start, int page_size,
+                                 int64_t page_stride, int B, int nh, int nkv, int hd, int window, float scale,
+                                 float softcap, const float* r1, const float* r2, int chunk, const float* sink,
+                                 void* out, float* partial, int decode, int max_new, int max_end, hipStream_t st) {
+  return tq_attention_mfma_wide_keys(q, k_pool, v_pool, block_table, bt_stride, cu_seqlens, slots, start, page_size,
+                                     page_stride, B, nh, nkv, hd, window, scale, softcap, r1, r2, chunk, sink, out, partial,
+                                     decode, max_new, max_end, 0, st);
 }
 
 TQ_API int tq_attention_mfma(const void* q, const void* k_pool, const void* v_pool, const int* block_table,

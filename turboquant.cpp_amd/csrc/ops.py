@@ -133,6 +133,9 @@ _OPTIONAL = {
                               _c_int, _c_int, _c_ptr],
     "tq_attention_mfma": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
                           _c_int, _c_int, _c_int, _c_f32, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "tq_attention_mfma_wide_keys": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int,
+                                    _c_int, _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr,
+                                    _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
 }
 
 
@@ -922,8 +925,11 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
               page_stride: int, num_heads: int, num_kv_heads: int, head_dim: int, window: int | None,
               scale: float, act, runs: dict | None = None, softcap: float | None = None,
               distance_bias: tuple[torch.Tensor, torch.Tensor] | None = None, chunk: int | None = None,
-              sink: torch.Tensor | None = None) -> torch.Tensor:
+              sink: torch.Tensor | None = None, value_width: int | None = None) -> torch.Tensor:
     """Each token attends to its sequence's cached positions up to its own; returns [T, nh*hd].
+
+    ``value_width``: a head's value rows hold zeros behind their first ``value_width`` numbers (keys wider than values, both
+    laid out at the keys' width); the output is zero there, and a kernel may leave those dimensions out.
 
     ``softcap`` c: a scaled score s becomes c tanh(s / c).  ``distance_bias`` (r1, r2), float32 [nh] each: then
     r1[h] ln(1 + r2[h] (i - j)) is taken off the score of query position i and key position j.  ``chunk`` n: position i
@@ -947,6 +953,7 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
     _need(num_heads % num_kv_heads == 0, k, "heads must be a multiple of kv heads")
     _need(head_dim <= 512, k, lambda: f"head size {head_dim} is beyond the 512 this kernel takes")
     _need(layer_offset + num_kv_heads * page_size * head_dim <= page_stride, k, "layer does not fit in a page")
+    _need(value_width is None or 1 <= value_width <= head_dim, k, "the values' width lies within the head")
     out = torch.empty_like(q)
     esz = k_pages.element_size()
     lib = library(act)
@@ -972,11 +979,12 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
             _need(T == B, k, "decoding brings one token per sequence")
             partial = torch.empty((lib.tq_attention_decode_scratch(B, num_heads, head_dim, int(runs["max_end"])),),
                                   dtype=torch.float32, device=q.device)
-        _run("attention_mfma", lib.tq_attention_mfma_mod(
+        _run("attention_mfma", lib.tq_attention_mfma_wide_keys(
             _ptr(q), k_pages.data_ptr() + layer_offset * esz, v_pages.data_ptr() + layer_offset * esz,
             _ptr(block_table), block_table.shape[1], _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]), _ptr(runs["start"]),
             page_size, page_stride, B, num_heads, num_kv_heads, head_dim, int(window or 0), float(scale), *mod, _ptr(out),
-            _ptr(partial), int(bool(runs["decode"])), int(runs["max_new"]), int(runs["max_end"]), _stream()))
+            _ptr(partial), int(bool(runs["decode"])), int(runs["max_new"]), int(runs["max_end"]), int(value_width or 0),
+            _stream()))
         return out
     if (runs is not None and dtype_name(act) == "float32" and hasattr(lib, "tq_attention_f32") and head_dim % 4 == 0
             and head_dim <= 256 and page_size % 64 == 0 and page_stride % 4 == 0 and layer_offset % 4 == 0):

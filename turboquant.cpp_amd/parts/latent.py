@@ -238,7 +238,8 @@ class LatentAttention(Part):
             queries = ops.rope_kv_write(q, b.positions, b.slot_of_token, table, *angles, None, None, 0, kv.page_size, stride,
                                         H, 0, D, ctx.act, runs=runs, amplitude=amp)
         mixed = ops.attention(queries, pages[0], pages[1], 0, b.positions, b.slot_of_token, table,
-                              kv.page_size, stride, H, H, D, None, self.scale, ctx.act, runs=runs)
+                              kv.page_size, stride, H, H, D, None, self.scale, ctx.act, runs=runs,
+                              value_width=-(-self.value_dim // 16) * 16)
         if gate is not None:
             ops.gate_rows(mixed, gate, self.gate_activation, ctx.act)
         return ops.gemm(mixed, self.out_weight, ctx.act, partial_sums=True)
