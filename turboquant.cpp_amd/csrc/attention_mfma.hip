@@ -61,6 +61,8 @@ struct AttnArgs {
   float* partial;               // decoding: [B][nh][max_runs][hd + 2]
   int max_runs;
   ScoreMod mod;                 // what happens to a score before the softmax, and the chunks of positions (score_mod.h)
+  const float* head_gate;       // null, or [T][ld_gate]: head h's output of token t is multiplied by sigmoid(head_gate[t][h])
+  int64_t ld_gate;
 };
 
 // What softmax_tile needs of the score's changes for the QG groups of columns a lane holds: the plain scale, the cap and
@@ -583,7 +585,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DT > 16 ? 1
 #pragma unroll
   for (int g = 0; g < QG; ++g) {
     if (p_q[g] < 0) continue;
-    const float inv = 1.0f / l_run[g];
+    float inv = 1.0f / l_run[g];
+    if (a.head_gate) inv /= 1.0f + expf(-a.head_gate[(size_t)(t0 + p_q[g] - start) * a.ld_gate + h]);
     bf16_t* orow = a.out + ((size_t)(t0 + p_q[g] - start) * a.nh + h) * hd;
 #pragma unroll
     for (int dt = 0; dt < VD; ++dt) {
@@ -698,7 +701,8 @@ __global__ __launch_bounds__(256) void attn_join_kernel(AttnArgs a) {
     l += wave_sum(wl);
   }
   __builtin_amdgcn_wave_barrier();
-  const float inv = 1.0f / l;
+  float inv = 1.0f / l;
+  if (a.head_gate) inv /= 1.0f + expf(-a.head_gate[(size_t)a.cu_seqlens[b] * a.ld_gate + h]);
   bf16_t* orow = a.out + ((size_t)a.cu_seqlens[b] * a.nh + h) * a.hd;
   if (a.hd % 128 == 0) {      // a lane takes two neighbouring dimensions of its wave's 128: one pass over the runs, 8 bytes at a time
     const int d = 128 * wave + 2 * lane;
@@ -769,22 +773,24 @@ TQ_API int64_t tq_attention_decode_scratch(int B, int nh, int hd, int max_end) {
 // max_end: largest position + 1 that any token of the step has.
 // softcap, r1, r2, chunk, sink: see score_mod.h (0, null, null, 0, null: nothing).
 // value_width (0: hd): the values' first numbers that matter; a head's value rows behind them are zeros, and so is the
-// output there, which lets a kernel leave them out.
-TQ_API int tq_attention_mfma_wide_keys(const void* q, const void* k_pool, const void* v_pool, const int* block_table,
+// output there, which lets a kernel leave them out.  head_gate (null: none), float [T][ld_gate]: the output of head h of
+// token t is multiplied by sigmoid(head_gate[t][h]) where it is normalised, before it is rounded.
+TQ_API int tq_attention_mfma_ex(const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                                        int bt_stride, const int* cu_seqlens, const int* slots, const int* start, int page_size,
                                        int64_t page_stride, int B, int nh, int nkv, int hd, int window, float scale,
                                        float softcap, const float* r1, const float* r2, int chunk, const float* sink,
                                        void* out, float* partial, int decode, int max_new, int max_end, int value_width,
-                                       hipStream_t st) {
+                                       const float* head_gate, int64_t ld_gate, hipStream_t st) {
   if (B <= 0) return 0;
-  if ((r1 == nullptr) != (r2 == nullptr) || chunk < 0 || softcap < 0.f || value_width < 0 || value_width > hd) return TQ_ERR_BAD_ARG;
+  if ((r1 == nullptr) != (r2 == nullptr) || chunk < 0 || softcap < 0.f || value_width < 0 || value_width > hd || (head_gate && ld_gate < nh))
+    return TQ_ERR_BAD_ARG;
   if (hd % 16 != 0 || hd < 16 || hd > 512 || page_size % TILE != 0 || nkv <= 0 || nh % nkv != 0)
     return TQ_ERR_UNSUPPORTED;
   if (nh > 65535 || B > 65535 || page_stride % 8 != 0 || !(scale > 0.f)) return TQ_ERR_UNSUPPORTED;
   if (decode && most_runs(max_end) > MAX_RUNS_LDS) return TQ_ERR_UNSUPPORTED;
   AttnArgs a{(const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, bt_stride, cu_seqlens, slots,
              start, page_size, page_stride, nh, nkv, hd, window, scale, (bf16_t*)out, partial,
-             most_runs(max_end), ScoreMod{softcap, r1, r2, chunk, sink}};
+             most_runs(max_end), ScoreMod{softcap, r1, r2, chunk, sink}, head_gate, ld_gate};
   const int dt = hd / 16;
   // head sizes 64, 128 and 256 have kernels of their own in which nothing depends on hd at run time
   if (decode) {
@@ -826,9 +832,9 @@ TQ_API int tq_attention_mfma_mod(const void* q, const void* k_pool, const void* 
                                  int64_t page_stride, int B, int nh, int nkv, int hd, int window, float scale,
                                  float softcap, const float* r1, const float* r2, int chunk, const float* sink,
                                  void* out, float* partial, int decode, int max_new, int max_end, hipStream_t st) {
-  return tq_attention_mfma_wide_keys(q, k_pool, v_pool, block_table, bt_stride, cu_seqlens, slots, start, page_size,
-                                     page_stride, B, nh, nkv, hd, window, scale, softcap, r1, r2, chunk, sink, out, partial,
-                                     decode, max_new, max_end, 0, st);
+  return tq_attention_mfma_ex(q, k_pool, v_pool, block_table, bt_stride, cu_seqlens, slots, start, page_size,
+                              page_stride, B, nh, nkv, hd, window, scale, softcap, r1, r2, chunk, sink, out, partial,
+                              decode, max_new, max_end, 0, nullptr, 0, st);
 }
 
 TQ_API int tq_attention_mfma(const void* q, const void* k_pool, const void* v_pool, const int* block_table,

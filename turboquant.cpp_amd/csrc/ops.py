@@ -133,9 +133,9 @@ _OPTIONAL = {
                               _c_int, _c_int, _c_ptr],
     "tq_attention_mfma": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
                           _c_int, _c_int, _c_int, _c_f32, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
-    "tq_attention_mfma_wide_keys": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int,
-                                    _c_int, _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr,
-                                    _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "tq_attention_mfma_ex": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int,
+                             _c_int, _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr,
+                             _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_i64, _c_ptr],
 }
 
 
@@ -925,11 +925,14 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
               page_stride: int, num_heads: int, num_kv_heads: int, head_dim: int, window: int | None,
               scale: float, act, runs: dict | None = None, softcap: float | None = None,
               distance_bias: tuple[torch.Tensor, torch.Tensor] | None = None, chunk: int | None = None,
-              sink: torch.Tensor | None = None, value_width: int | None = None) -> torch.Tensor:
+              sink: torch.Tensor | None = None, value_width: int | None = None,
+              head_gate: torch.Tensor | None = None) -> torch.Tensor:
     """Each token attends to its sequence's cached positions up to its own; returns [T, nh*hd].
 
     ``value_width``: a head's value rows hold zeros behind their first ``value_width`` numbers (keys wider than values, both
     laid out at the keys' width); the output is zero there, and a kernel may leave those dimensions out.
+    ``head_gate`` float32 [T, nh] (rows may be runs of columns of a wider tensor): head h's output of token t is multiplied by
+    sigmoid(head_gate[t, h]), in the kernel that normalises the output where it knows how, else by ``gate_heads`` behind it.
 
     ``softcap`` c: a scaled score s becomes c tanh(s / c).  ``distance_bias`` (r1, r2), float32 [nh] each: then
     r1[h] ln(1 + r2[h] (i - j)) is taken off the score of query position i and key position j.  ``chunk`` n: position i
@@ -954,6 +957,9 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
     _need(head_dim <= 512, k, lambda: f"head size {head_dim} is beyond the 512 this kernel takes")
     _need(layer_offset + num_kv_heads * page_size * head_dim <= page_stride, k, "layer does not fit in a page")
     _need(value_width is None or 1 <= value_width <= head_dim, k, "the values' width lies within the head")
+    _need(head_gate is None or (isinstance(head_gate, torch.Tensor) and head_gate.is_cuda and head_gate.dtype == torch.float32
+                                and tuple(head_gate.shape) == (T, num_heads) and head_gate.stride(1) == 1), k,
+          lambda: f"head_gate must be float32 [{T}, {num_heads}] on the GPU with unit stride along its rows")
     out = torch.empty_like(q)
     esz = k_pages.element_size()
     lib = library(act)
@@ -979,12 +985,12 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
             _need(T == B, k, "decoding brings one token per sequence")
             partial = torch.empty((lib.tq_attention_decode_scratch(B, num_heads, head_dim, int(runs["max_end"])),),
                                   dtype=torch.float32, device=q.device)
-        _run("attention_mfma", lib.tq_attention_mfma_wide_keys(
+        _run("attention_mfma", lib.tq_attention_mfma_ex(
             _ptr(q), k_pages.data_ptr() + layer_offset * esz, v_pages.data_ptr() + layer_offset * esz,
             _ptr(block_table), block_table.shape[1], _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]), _ptr(runs["start"]),
             page_size, page_stride, B, num_heads, num_kv_heads, head_dim, int(window or 0), float(scale), *mod, _ptr(out),
             _ptr(partial), int(bool(runs["decode"])), int(runs["max_new"]), int(runs["max_end"]), int(value_width or 0),
-            _stream()))
+            _ptr(head_gate), head_gate.stride(0) if head_gate is not None else 0, _stream()))
         return out
     if (runs is not None and dtype_name(act) == "float32" and hasattr(lib, "tq_attention_f32") and head_dim % 4 == 0
             and head_dim <= 256 and page_size % 64 == 0 and page_stride % 4 == 0 and layer_offset % 4 == 0):
@@ -1003,13 +1009,13 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
             _ptr(block_table), block_table.shape[1], _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]), _ptr(runs["start"]),
             page_size, page_stride, B, num_heads, num_kv_heads, head_dim, int(window or 0), float(scale), *mod, _ptr(out),
             _ptr(partial), int(bool(runs["decode"])), int(runs["max_new"]), int(runs["max_end"]), _stream()))
-        return out
+        return out if head_gate is None else gate_heads(out, head_gate, num_heads, "sigmoid", act)
     _run(k, lib.tq_attention_generic_mod(_ptr(q), k_pages.data_ptr() + layer_offset * esz,
                                          v_pages.data_ptr() + layer_offset * esz, _ptr(positions),
                                          _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], page_size,
                                          page_stride, T, num_heads, num_kv_heads, head_dim, int(window or 0),
                                          float(scale), *mod, _ptr(out), _stream()))
-    return out
+    return out if head_gate is None else gate_heads(out, head_gate, num_heads, "sigmoid", act)
 
 
 # ------------------------------------------------------------------ routing

@@ -101,11 +101,11 @@ int tq_attention_mfma_mod(const void* q, const void* k_pool, const void* v_pool,
         const int* cu_seqlens, const int* slots, const int* start, int page_size, int64_t page_stride, int B,
         int nh, int nkv, int hd, int window, float scale, float softcap, const float* r1, const float* r2, int chunk,
         const float* sink, void* out, float* partial, int decode, int max_new, int max_end, hipStream_t st);
-int tq_attention_mfma_wide_keys(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
+int tq_attention_mfma_ex(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
         const int* cu_seqlens, const int* slots, const int* start, int page_size, int64_t page_stride, int B,
         int nh, int nkv, int hd, int window, float scale, float softcap, const float* r1, const float* r2, int chunk,
         const float* sink, void* out, float* partial, int decode, int max_new, int max_end, int value_width,
-        hipStream_t st);
+        const float* head_gate, int64_t ld_gate, hipStream_t st);
 // attention_f32.hip: float32 attention on the matrix cores (float32 library)
 int64_t tq_attention_f32_scratch(int B, int nh, int hd, int max_end);
 int tq_attention_f32(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,

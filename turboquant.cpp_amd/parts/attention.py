@@ -228,7 +228,7 @@ class GroupedQueryAttention(Part):
     def _forward_extended(self, normed, ctx, b, kv, amplitude):
         """The forms with a norm behind the rotation, scaled sines and cosines, a gate per head or another layer's keys
         and values: one product of the layer's input (q | k | v | gate rows), the rotation with its norm and the cache
-        write in one launch, attention, the gate, the output product."""
+        write in one launch, attention with the gate where it normalises its output, the output product."""
         if kv.owns == self.shares_kv:
             raise ValueError("an attention keeps a cache of its own exactly if it has keys and values of its own")
         H, G, D = self.num_heads, 0 if self.shares_kv else self.num_kv_heads, self.head_dim
@@ -246,7 +246,6 @@ class GroupedQueryAttention(Part):
                               runs=b.runs(), amplitude=amplitude, norm_eps=self.rotated_norm_eps, norm_dim=self.key_dim)
         o = ops.attention(q, kv.k_pages, kv.v_pages, kv.layer_offset, b.positions, b.slot_of_token, kv.table,
                           kv.page_size, kv.page_stride, H, self.num_kv_heads, D, self.window, self.scale, ctx.act,
-                          runs=b.runs(), **self._score_options())
-        if self.has_head_gate:
-            ops.gate_heads(o, proj[:, width:width + H], H, "sigmoid", ctx.act)
+                          runs=b.runs(), head_gate=proj[:, width:width + H] if self.has_head_gate else None,
+                          **self._score_options())
         return ops.gemm(o, self.out_weight, ctx.act, bias=self.out_bias, partial_sums=True)
