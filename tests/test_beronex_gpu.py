@@ -551,7 +551,8 @@ def test_a_gate_per_head_and_a_norm_of_a_row_s_first_part():
             got = ops.gate_heads(f32(o).to(dt), f32(g)[:, 2:2 + H], H, "sigmoid", act)
             want = (o.reshape(M, H, hd) * plain.sigmoid(g[:, 2:2 + H])[:, :, None]).reshape(M, H * hd)
             assert np.abs(got.double().cpu().numpy() - want).max() < tol * max(1.0, np.abs(want).max())
-    for T, R, lead, width, copies in ((1, 20, 4, 32, 2), (70, 80, 16, 96, 3), (9, 304, 0, 304, 1), (33, 18, 6, 32, 2)):
+    for T, R, lead, width, copies in ((1, 20, 4, 32, 2), (70, 80, 16, 96, 3), (9, 304, 0, 304, 1), (33, 18, 6, 32, 2),
+                                         (1, 700, 64, 768, 2), (32, 130, 2, 144, 3), (33, 300, 8, 320, 1)):
         src, wt = rng.normal(size=(T, R + lead + 7)), rng.normal(1, 0.1, R)
         got = ops.lead_norm(f32(src)[:, 3:3 + R + lead], R, f32(wt), 1e-5, copies, width, "float32").double().cpu().numpy()
         want = plain.rms_norm(src[:, 3:3 + R], wt, 1e-5)

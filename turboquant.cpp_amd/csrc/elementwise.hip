@@ -424,11 +424,47 @@ __global__ __launch_bounds__(256) void lead_norm_kernel(const float* __restrict_
   }
 }
 
+// The same for steps of a few tokens, a workgroup to a token: a wave alone walks a row of several hundred numbers in a
+// dozen dependent rounds.
+template <class W, class O>
+__global__ __launch_bounds__(256) void lead_norm_few_kernel(const float* __restrict__ in, int64_t ld_in, const W* __restrict__ w,
+                                                            float eps, O* __restrict__ out, int64_t ld_out, int copies, int R,
+                                                            int lead, int Rp) {
+  __shared__ float part[256 / TQ_WAVE];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const float* row = in + (size_t)t * ld_in;
+  float ss = 0.f;
+  for (int i = tid; i < R; i += 256) ss += row[i] * row[i];
+  ss = wave_sum(ss);
+  if (tid % TQ_WAVE == 0) part[tid / TQ_WAVE] = ss;
+  __syncthreads();
+  ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 256 / TQ_WAVE; ++i) ss += part[i];
+  const float rs = 1.0f / sqrtf(ss / (float)R + eps);
+  for (int i = tid; i < Rp; i += 256) {
+    const float v = i < lead ? row[R + i] : i < lead + R ? row[i - lead] * rs * to_f32(w[i - lead]) : 0.f;
+    for (int c = 0; c < copies; ++c) out[(size_t)t * ld_out + (size_t)c * Rp + i] = from_f32<O>(v);
+  }
+}
+
 TQ_API int tq_lead_norm(const float* in, int64_t ld_in, const void* w, int wtype, float eps, void* out, int out_is_act,
                         int64_t ld_out, int copies, int R, int lead, int Rp, int T, hipStream_t st) {
   if (T <= 0) return 0;
   if (R < 1 || lead < 0 || Rp < R + lead || copies < 1 || ld_in < R + lead || ld_out < (int64_t)copies * Rp || !w)
     return TQ_ERR_BAD_ARG;
+  if (T <= 32 && R > 2 * TQ_WAVE) {
+    TQ_DISPATCH_W(wtype, {
+      if (out_is_act)
+        hipLaunchKernelGGL((lead_norm_few_kernel<W, act_t>), dim3(T), dim3(256), 0, st, in, ld_in, (const W*)w, eps,
+                           (act_t*)out, ld_out, copies, R, lead, Rp);
+      else
+        hipLaunchKernelGGL((lead_norm_few_kernel<W, float>), dim3(T), dim3(256), 0, st, in, ld_in, (const W*)w, eps,
+                           (float*)out, ld_out, copies, R, lead, Rp);
+    });
+    TQ_LAUNCH_CHECK();
+    return 0;
+  }
   TQ_DISPATCH_W(wtype, {
     if (out_is_act)
       hipLaunchKernelGGL((lead_norm_kernel<W, act_t>), dim3((T + 3) / 4), dim3(256), 0, st, in, ld_in, (const W*)w, eps,
