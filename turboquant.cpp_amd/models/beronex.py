@@ -122,8 +122,8 @@ def _rotation(m: dict, where: str, width: int) -> Rotation | None:
         return Rotation(dims, base)
     s = KeyReader(scaling, where + ".rot.scaling")
     values = (s.number("factor"), s.number("original"), s.number("fast"), s.number("slow"))
-    require(values[0] >= 1 and min(values[1:]) > 0 and base > 1,
-            f"{where}.rot.scaling: factor must be at least 1, original, fast and slow positive, base above 1")
+    require(min(values) > 0 and base != 1,
+            f"{where}.rot.scaling: factor, original, fast and slow must be positive, and base other than 1")
     return Rotation(dims, base, tuple(float(v) for v in values))
 
 
@@ -133,6 +133,8 @@ def _mixer(kind: str, m: dict, where: str, index: int, n_layers: int):
     dim, vdim = r.integer("dim", minimum=1), r.integer("vdim", minimum=1)
     if kind == LIGHTNING:
         decay = m.get("decay")
+        if isinstance(decay, (int, float)) and not isinstance(decay, bool):      # one number: the same for every head
+            decay = [decay] * heads
         require(isinstance(decay, list) and len(decay) == heads
                 and all(isinstance(d, (int, float)) and not isinstance(d, bool) and 0 <= d <= 1 for d in decay),
                 f"{where}: decay must list a number between 0 and 1 for each of the {heads} heads")

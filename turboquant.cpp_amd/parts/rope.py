@@ -89,8 +89,8 @@ class YarnRotaryEncoding(RotaryEncoding):
     def __init__(self, head_dim: int, rotary_dim: int, theta: float, factor: float, original: float, fast: float,
                  slow: float, pairing: str = "half"):
         super().__init__(head_dim, rotary_dim, theta, pairing)
-        if not (factor >= 1.0 and original > 0 and fast > 0 and slow > 0 and theta > 1.0):
-            raise ValueError("YaRN needs factor >= 1, theta > 1 and positive original, fast and slow")
+        if not (factor > 0 and original > 0 and fast > 0 and slow > 0 and theta > 0 and theta != 1.0):
+            raise ValueError("YaRN needs a theta other than 1 and positive factor, theta, original, fast and slow")
         self.factor, self.original, self.fast, self.slow = float(factor), float(original), float(fast), float(slow)
         self.amplitude = 0.1 * math.log(self.factor) + 1.0
 
