@@ -77,6 +77,7 @@ class GroupKey:
     value_dim: int
     window: int | None
     chunk: int | None = None
+    keep_first: int = 0
 
 
 @dataclass
@@ -134,6 +135,17 @@ class CacheGroup:
         if self.key.chunk is not None:      # the token at position `length` and all later ones see its chunk's start at the earliest
             first = max(first, length // self.key.chunk * self.key.chunk)
         return first // self.page_size
+
+    @property
+    def kept_pages(self) -> int:
+        """Logical pages from the start that hold positions every later token sees: they are never given back."""
+        return -(-self.key.keep_first // self.page_size)
+
+    def needed_pages(self, length: int) -> list[int]:
+        """The logical pages that a sequence of ``length`` positions holds after a commit, in ascending order."""
+        last = (length - 1) // self.page_size if length else -1
+        first = self.first_needed_page(length)
+        return [p for p in range(last + 1) if p >= first or p < self.kept_pages]
 
     def sync(self) -> None:
         """Sends the rows of the page table that changed to the device.  On a GPU they go through pinned memory
@@ -202,7 +214,8 @@ class PagedCache:
         for e, (cache_need, _state, cache_of) in enumerate(self._needs):
             if cache_need is not None and cache_of is None:
                 by_key.setdefault(GroupKey(cache_need.num_kv_heads, cache_need.head_dim, cache_need.value_width,
-                                           cache_need.window, cache_need.chunk), []).append(e)
+                                           cache_need.window, cache_need.chunk,
+                                           cache_need.keep_first if cache_need.window is not None else 0), []).append(e)
         # A sequence holds, of a group with a window, the pages that its last `window` positions touch, and during a
         # step those of the step's new positions too, until the step is committed: window + window_step positions
         # lie in at most that many pages plus two.
@@ -211,7 +224,7 @@ class PagedCache:
         for key, entries in by_key.items():
             pages = self.n_pages
             if key.window is not None:
-                for_windows = self.max_slots * (-(-(key.window + window_step) // page_size) + 2)
+                for_windows = self.max_slots * (-(-(key.window + window_step) // page_size) + 2 + -(-key.keep_first // page_size))
                 if for_windows < pages:
                     pages, self.step_limit = for_windows, window_step
             self.groups.append(CacheGroup(key, entries, pages, page_size, self.max_slots, per_seq, dtype, device))
@@ -231,6 +244,8 @@ class PagedCache:
                     raise CacheError(f"schedule entry {e} reads the cache of entry {cache_of} but their head counts or sizes differ")
                 if src.window is not None and (cache_need.window is None or cache_need.window > src.window):
                     raise CacheError(f"schedule entry {e} looks further back than entry {cache_of}, whose cache it reads, keeps")
+                if src.window is not None and cache_need.keep_first > src.keep_first:
+                    raise CacheError(f"schedule entry {e} keeps more first positions in sight than entry {cache_of}, whose cache it reads, keeps")
                 if src.chunk is not None and cache_need.chunk != src.chunk:
                     raise CacheError(f"schedule entry {e} reads the cache of entry {cache_of}, which keeps chunks of {src.chunk} positions only")
                 self._entry_group[e] = (g, off, False)
@@ -359,7 +374,7 @@ class PagedCache:
             first = g.first_needed_page(s.length)
             if first > 0:
                 row = g.host_table[slot]
-                old = [p for p in range(first) if row[p] >= 0]
+                old = [p for p in range(g.kept_pages, first) if row[p] >= 0]
                 if old:
                     g.pool.give_back(row[old].tolist())
                     row[old] = -1
@@ -379,14 +394,14 @@ class PagedCache:
             return
         if any(state is not None for _c, state, _o in self._needs):
             raise CacheError("a model with fixed-size state per sequence cannot go back to an earlier position")
-        last = (length - 1) // self.page_size if length else -1
         for g in self.groups:
             row = g.host_table[slot]
-            if any(row[p] < 0 for p in range(g.first_needed_page(length), last + 1)):
+            if any(row[p] < 0 for p in g.needed_pages(length)):
                 raise CacheError(f"the window of a group has given back pages that position {length} would look at")
         for g in self.groups:
             row = g.host_table[slot]
-            gone = [p for p in range(g.max_pages_per_seq) if row[p] >= 0 and (p > last or p < g.first_needed_page(length))]
+            needed = set(g.needed_pages(length))
+            gone = [p for p in range(g.max_pages_per_seq) if row[p] >= 0 and p not in needed]
             if gone:
                 g.pool.give_back(row[gone].tolist())
                 row[gone] = -1
@@ -400,15 +415,14 @@ class PagedCache:
         if s.reserved:
             raise CacheError(f"slot {slot} has positions reserved for a running step")
         out = {"length": s.length, "page_size": self.page_size, "groups": [], "states": {}}
-        last = (s.length - 1) // self.page_size if s.length else -1
         for g in self.groups:
             first = g.first_needed_page(s.length)
             row = g.host_table[slot]
-            pages = [int(row[p]) for p in range(first, last + 1)]
+            pages = [int(row[p]) for p in g.needed_pages(s.length)]
             if any(p < 0 for p in pages):
                 raise CacheError(f"slot {slot} does not hold all pages of its {s.length} positions")
             idx = torch.tensor(pages, dtype=torch.int64, device=self.device)
-            entry = {"first_page": first, "entries": list(g.entries), "key": (g.key.num_kv_heads, g.key.head_dim, g.key.value_dim, g.key.window, g.key.chunk),
+            entry = {"first_page": first, "entries": list(g.entries), "key": (g.key.num_kv_heads, g.key.head_dim, g.key.value_dim, g.key.window, g.key.chunk, g.key.keep_first),
                      "keys": g.k_pages.view(-1, g.page_stride)[idx].cpu(), "values": None}
             if g.v_pages is not None:
                 entry["values"] = g.v_pages.view(-1, g.v_page_stride)[idx].cpu()
@@ -422,7 +436,10 @@ class PagedCache:
         if data["page_size"] != self.page_size or len(data["groups"]) != len(self.groups):
             raise CacheError("the saved sequence comes from a cache of another layout")
         for g, d in zip(self.groups, data["groups"]):
-            if tuple(d["key"]) + (None,) * (5 - len(d["key"])) != (g.key.num_kv_heads, g.key.head_dim, g.key.value_dim, g.key.window, g.key.chunk) or \
+            saved = tuple(d["key"])
+            saved += (None,) * (5 - len(saved))
+            saved += (0,) * (6 - len(saved))
+            if saved != (g.key.num_kv_heads, g.key.head_dim, g.key.value_dim, g.key.window, g.key.chunk, g.key.keep_first) or \
                     list(d["entries"]) != list(g.entries) or d["keys"].dtype != self.dtype or \
                     d["keys"].shape[1] != g.page_stride or (d["values"] is None) != (g.v_pages is None):
                 raise CacheError("the saved sequence comes from a cache of another layout")
@@ -432,13 +449,13 @@ class PagedCache:
             if length:
                 self.reserve(slot, length)
                 self.commit(slot)
-            last = (length - 1) // self.page_size if length else -1
             for g, d in zip(self.groups, data["groups"]):
                 first = g.first_needed_page(length)
-                if d["first_page"] != first or d["keys"].shape[0] != last + 1 - first:
+                needed = g.needed_pages(length)
+                if d["first_page"] != first or d["keys"].shape[0] != len(needed):
                     raise CacheError("the saved pages do not cover the saved length")
                 row = g.host_table[slot]
-                idx = torch.tensor([int(row[p]) for p in range(first, last + 1)], dtype=torch.int64, device=self.device)
+                idx = torch.tensor([int(row[p]) for p in needed], dtype=torch.int64, device=self.device)
                 if idx.numel():
                     g.k_pages.view(-1, g.page_stride)[idx] = d["keys"].to(self.device)
                     if g.v_pages is not None:

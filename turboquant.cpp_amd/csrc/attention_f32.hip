@@ -75,7 +75,7 @@ __device__ __forceinline__ float group_sum(float v) {
 // update, and the product with the values from `vf` (value operand of d-tile dt, subtile kt).
 template <int ND, class KF, class VF>
 __device__ __forceinline__ void attend_tile(const f32x4 (&qf)[ND], KF kf, VF vf, int key0, int pos_q, int lo_q, float scale,
-                                            float cap, bool biased, float r1, float r2,
+                                            float cap, bool biased, float r1, float r2, int keep, bool sig, float pb,
                                             float& m_run, float& l_run, f32x4 (&acc)[ND]) {
   const int g = (threadIdx.x % 64) / 16;
   f32x4 s[4];
@@ -95,11 +95,11 @@ __device__ __forceinline__ void attend_tile(const f32x4 (&qf)[ND], KF kf, VF vf,
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       const int j = key0 + 16 * kt + 4 * g + v;
-      const float x = (j <= pos_q && j >= lo_q) ? mod_score(s[kt][v] * scale, cap, biased, r1, r2, pos_q - j) : -INFINITY;
+      const float x = sees(j, pos_q, lo_q, keep) ? mod_score(s[kt][v] * scale, cap, biased, r1, r2, pos_q - j) : -INFINITY;
       s[kt][v] = x;
       m_tile = fmaxf(m_tile, x);
     }
-  m_tile = group_max(m_tile);
+  m_tile = sig ? 0.f : group_max(m_tile);      // sigmoid weights: the maximum stays where it starts, at 0
   // (a query that has nothing in its reach so far keeps a maximum of -inf: its probabilities and its factor for what
   // came before are 0 below, never exp(-inf + inf); all lanes stay together for the matrix instructions)
   const float m_new = fmaxf(m_run, m_tile);
@@ -108,7 +108,7 @@ __device__ __forceinline__ void attend_tile(const f32x4 (&qf)[ND], KF kf, VF vf,
   for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      const float p = s[kt][v] == -INFINITY ? 0.f : expf(s[kt][v] - m_new);
+      const float p = s[kt][v] == -INFINITY ? 0.f : (sig ? sigmoid_weight(s[kt][v] + pb) : expf(s[kt][v] - m_new));
       s[kt][v] = p;
       l_tile += p;
     }
@@ -168,6 +168,10 @@ __global__ __launch_bounds__(256) void attn_f32_prefill_kernel(AttnF32Args p, in
     m_run = p.mod.sink[h];
     l_run = 1.f;
   }
+  const bool sig = p.mod.pb != nullptr;
+  const float pb = sig ? p.mod.pb[h] : 0.f;
+  if (sig) m_run = 0.f;
+  const int keep = p.mod.keep, kept = keep_tiles(keep, AT);
 
   // what the block as a whole can reach, and what this wave can
   const int blk_first = start + blk * 64, blk_last = start + min(n_new, blk * 64 + 64) - 1;
@@ -175,7 +179,7 @@ __global__ __launch_bounds__(256) void attn_f32_prefill_kernel(AttnF32Args p, in
   const int wave_first = start + blk * 64 + wave * 16, wave_last = min(blk_last, wave_first + 15);
   const int wave_lo = reach_lo(wave_first, p.window, p.mod.chunk);
 
-  for (int tile = blk_lo / AT; tile * AT <= blk_last; ++tile) {
+  for (int tile = first_tile(blk_lo / AT, kept); tile * AT <= blk_last; tile = next_tile(tile, blk_lo / AT, kept)) {
     const int key0 = tile * AT;
     const int page = table[key0 / p.page_size];
     __syncthreads();          // the tile before has been used by every wave
@@ -194,14 +198,14 @@ __global__ __launch_bounds__(256) void attn_f32_prefill_kernel(AttnF32Args p, in
     }
     __syncthreads();
     if (page < 0) continue;             // a page that its group has given back: nothing of it is in anyone's reach
-    if (key0 > wave_last || key0 + AT <= wave_lo) continue;
+    if (key0 > wave_last || (key0 + AT <= wave_lo && key0 >= keep)) continue;
     attend_tile<ND>(
         qf, [&](int kt, int u) { return *reinterpret_cast<const f32x4*>(&Ks[(16 * kt + r) * KLD + 16 * u + 4 * g]); },
         [&](int dt, int kt) { return *reinterpret_cast<const f32x4*>(&Vt[(16 * dt + r) * VLD + 16 * kt + 4 * g]); },
-        key0, pos_q, lo_q, p.scale, p.mod.cap, biased, r1, r2, m_run, l_run, acc);
+        key0, pos_q, lo_q, p.scale, p.mod.cap, biased, r1, r2, keep, sig, pb, m_run, l_run, acc);
   }
   if (!q_ok) return;
-  const float inv = 1.0f / l_run;
+  const float inv = sig ? 1.0f : 1.0f / l_run;
   float* orow = p.out + ((size_t)(t0 + qi) * p.nh + h) * hd;
 #pragma unroll
   for (int dt = 0; dt < ND; ++dt) {
@@ -227,8 +231,10 @@ __global__ __launch_bounds__(64) void attn_f32_decode_kernel(AttnF32Args p, int 
   const int lane = threadIdx.x, r = lane % 16, g = lane / 16;
   const int pos = p.start[b];                       // the token's position: it attends to lo..pos
   const int lo = reach_lo(pos, p.window, p.mod.chunk);
-  const int first = lo / AT, last = pos / AT;
-  const int tile = first + blockIdx.z;
+  int first = lo / AT, kept = keep_tiles(p.mod.keep, AT);
+  const int last = pos / AT;
+  if (first <= kept) first = kept = 0;        // the window reaches the kept tiles: one run of tiles from the start
+  const int tile = (int)blockIdx.z < kept ? (int)blockIdx.z : first + (int)blockIdx.z - kept;
   if (tile > last) return;
   const int* table = p.block_table + (size_t)p.slots[b] * p.bt_stride;
   const int hd = p.hd, group = p.nh / p.nkv;
@@ -253,7 +259,9 @@ __global__ __launch_bounds__(64) void attn_f32_decode_kernel(AttnF32Args p, int 
     f32x4 acc[ND];
 #pragma unroll
     for (int dt = 0; dt < ND; ++dt) acc[dt] = zero;
-    float m_run = -INFINITY, l_run = 0.f;
+    const bool sig = p.mod.pb != nullptr;
+    const float pb = sig ? p.mod.pb[h] : 0.f;
+    float m_run = sig ? 0.f : -INFINITY, l_run = 0.f;
     const float* kp = p.k_pool + (size_t)page * p.page_stride + ((size_t)kvh * p.page_size + key0 % p.page_size) * hd;
     const float* vp = p.v_pool + (size_t)page * p.page_stride + (size_t)kvh * p.page_size * hd + key0 % p.page_size;
     if (LINES) {
@@ -279,7 +287,7 @@ __global__ __launch_bounds__(64) void attn_f32_decode_kernel(AttnF32Args p, int 
             v_next = t1;
             return t0;
           },
-          key0, q_ok ? pos : -1, lo, p.scale, p.mod.cap, biased, r1, r2, m_run, l_run, acc);
+          key0, q_ok ? pos : -1, lo, p.scale, p.mod.cap, biased, r1, r2, p.mod.keep, sig, pb, m_run, l_run, acc);
     } else {
       // (what lies beyond the head size is asked for at the tile's first address instead and replaced by zeros:
       // every lane loads, so that no load waits behind a branch)
@@ -296,7 +304,7 @@ __global__ __launch_bounds__(64) void attn_f32_decode_kernel(AttnF32Args p, int 
                 reinterpret_cast<const f32x4*>(d < hd ? vp + (size_t)d * p.page_size + 16 * kt + 4 * g : vp));
             return d < hd ? x : zero;
           },
-          key0, q_ok ? pos : -1, lo, p.scale, p.mod.cap, biased, r1, r2, m_run, l_run, acc);
+          key0, q_ok ? pos : -1, lo, p.scale, p.mod.cap, biased, r1, r2, p.mod.keep, sig, pb, m_run, l_run, acc);
     }
     if (!q_ok) return;
     float* out = p.partial + (((size_t)b * p.nh + h) * p.tiles_max + tile) * (hd + 2);
@@ -324,37 +332,42 @@ __global__ __launch_bounds__(64) void attn_f32_join_kernel(AttnF32Args p) {
   const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int pos = p.start[b];
   const int lo = reach_lo(pos, p.window, p.mod.chunk);
-  const int first = lo / AT, last = pos / AT;
+  int first = lo / AT, kept = keep_tiles(p.mod.keep, AT);
+  const int last = pos / AT;
+  if (first <= kept) first = kept = 0;
+  const int n_tiles = kept + last - first + 1;       // the kept tiles, then the window's: entry i is tile tile_of(i)
+#define TILE_OF(i) ((i) < kept ? (i) : first + (i) - kept)
   const int stride = p.hd + 2;
   const float* part = p.partial + ((size_t)b * p.nh + h) * p.tiles_max * stride;
   float m = -INFINITY;
-  for (int tile = first + lane; tile <= last; tile += 64) m = fmaxf(m, part[(size_t)tile * stride]);
+  for (int i = lane; i < n_tiles; i += 64) m = fmaxf(m, part[(size_t)TILE_OF(i) * stride]);
   m = wave_max(m);
   float l = 0.f;
   if (p.mod.sink) {         // the sink joins here, once, like one more tile with a sum of 1 and no values
     m = fmaxf(m, p.mod.sink[h]);
     l = expf(p.mod.sink[h] - m);
   }
-  for (int t0 = first; t0 <= last; t0 += 64) {
-    const int tile = t0 + lane;
+  for (int i0 = 0; i0 < n_tiles; i0 += 64) {
+    const int i = i0 + lane;
     float w = 0.f, wl = 0.f;
-    if (tile <= last) {
-      const float* q = part + (size_t)tile * stride;
+    if (i < n_tiles) {
+      const float* q = part + (size_t)TILE_OF(i) * stride;
       w = expf(q[0] - m);
       wl = w * q[1];
-      wgt[tile - first] = w;
+      wgt[i] = w;
     }
     l += wave_sum(wl);
   }
   __builtin_amdgcn_wave_barrier();
-  const float inv = 1.0f / l;
+  const float inv = p.mod.pb ? 1.0f : 1.0f / l;       // sigmoid weights are not normalised (every tile's maximum is 0)
   float* orow = p.out + ((size_t)p.cu_seqlens[b] * p.nh + h) * p.hd;
   for (int d = lane; d < p.hd; d += 64) {
     float a = 0.f;
 #pragma unroll 8
-    for (int tile = first; tile <= last; ++tile) a = fmaf(wgt[tile - first], part[(size_t)tile * stride + 2 + d], a);
+    for (int i = 0; i < n_tiles; ++i) a = fmaf(wgt[i], part[(size_t)TILE_OF(i) * stride + 2 + d], a);
     orow[d] = a * inv;
   }
+#undef TILE_OF
 }
 
 // Floats of `partial` that a decode step of B sequences up to max_end positions needs.
@@ -370,6 +383,7 @@ static int launch_attention_f32(const AttnF32Args& p, int B, int decode, int max
     // with a window a token reaches at most window positions, which lie in window / AT + 2 tiles at the most
     int waves = p.window > 0 ? min(tiles, p.window / AT + 2) : tiles;
     if (p.mod.chunk > 0) waves = min(waves, p.mod.chunk / AT + 2);      // and a chunk in chunk / AT + 2
+    waves = min(tiles, waves + keep_tiles(p.mod.keep, AT));              // and the kept first positions in tiles of their own
     if (p.nkv * passes > 65535 || waves > 65535 || tiles > F32_JOIN_TILES) return TQ_ERR_UNSUPPORTED;
     // whole lines only where the head fills its tiles of 16 (32, 64, 128, 256): the loads of that form have no
     // guard on the head size, and a head of 96 would read beyond its rows and, in the last page, beyond the pool
@@ -394,6 +408,12 @@ static int launch_attention_f32(const AttnF32Args& p, int B, int decode, int max
   return 0;
 }
 
+TQ_API int tq_attention_f32_sig(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
+                                const int* cu_seqlens, const int* slots, const int* start, int page_size, int64_t page_stride,
+                                int B, int nh, int nkv, int hd, int window, float scale, float softcap, const float* r1,
+                                const float* r2, int chunk, const float* sink, const float* pb, int keep, void* out,
+                                void* partial, int decode, int max_new, int max_end, hipStream_t st);
+
 // The tokens are runs of consecutive positions, one per sequence (cu_seqlens, slots, start as in AttnF32Args);
 // decode: every run is one token and `partial` holds tq_attention_f32_scratch(B, nh, hd, max_end) floats.
 // hd must be a multiple of 4 and at most 256, page_size a multiple of 64, page_stride a multiple of 4.
@@ -403,8 +423,19 @@ TQ_API int tq_attention_f32_mod(const void* q, const void* k_pool, const void* v
                                 int B, int nh, int nkv, int hd, int window, float scale, float softcap, const float* r1,
                                 const float* r2, int chunk, const float* sink, void* out, void* partial, int decode,
                                 int max_new, int max_end, hipStream_t st) {
+  return tq_attention_f32_sig(q, k_pool, v_pool, block_table, bt_stride, cu_seqlens, slots, start, page_size, page_stride, B,
+                              nh, nkv, hd, window, scale, softcap, r1, r2, chunk, sink, nullptr, 0, out, partial, decode,
+                              max_new, max_end, st);
+}
+
+// pb, keep: sigmoid weights with a bias per head, and first positions that stay visible (score_mod.h; null, 0: neither).
+TQ_API int tq_attention_f32_sig(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
+                                const int* cu_seqlens, const int* slots, const int* start, int page_size, int64_t page_stride,
+                                int B, int nh, int nkv, int hd, int window, float scale, float softcap, const float* r1,
+                                const float* r2, int chunk, const float* sink, const float* pb, int keep, void* out,
+                                void* partial, int decode, int max_new, int max_end, hipStream_t st) {
   if (B <= 0) return 0;
-  if ((r1 == nullptr) != (r2 == nullptr) || chunk < 0 || softcap < 0.f) return TQ_ERR_BAD_ARG;
+  if ((r1 == nullptr) != (r2 == nullptr) || chunk < 0 || softcap < 0.f || keep < 0 || (pb && sink)) return TQ_ERR_BAD_ARG;
   if (hd <= 0 || hd % 4 != 0 || hd > 256 || nkv <= 0 || nh % nkv != 0 || page_size % AT != 0 || page_stride % 4 != 0)
     return TQ_ERR_UNSUPPORTED;
   if (((size_t)q | (size_t)k_pool | (size_t)v_pool | (size_t)out) & 15) return TQ_ERR_UNSUPPORTED;
@@ -412,7 +443,7 @@ TQ_API int tq_attention_f32_mod(const void* q, const void* k_pool, const void* v
   if (max_new <= 0 || max_end <= 0) return TQ_ERR_BAD_ARG;
   AttnF32Args p{(const float*)q, (const float*)k_pool, (const float*)v_pool, block_table, bt_stride, cu_seqlens, slots,
                 start, page_size, page_stride, nh, nkv, hd, window, scale, (float*)out, (float*)partial,
-                (max_end + AT - 1) / AT, ScoreMod{softcap, r1, r2, chunk, sink}};
+                (max_end + AT - 1) / AT, ScoreMod{softcap, r1, r2, chunk, sink, pb, keep}};
   int rc;
   if (hd <= 16) rc = launch_attention_f32<1>(p, B, decode, max_new, max_end, st);
   else if (hd <= 32) rc = launch_attention_f32<2>(p, B, decode, max_new, max_end, st);

@@ -44,10 +44,15 @@ __global__ __launch_bounds__(CHUNK) void attention_generic_kernel(
     m_run = mod.sink[h];
     l_run = 1.f;
   }
+  const bool sig = mod.pb != nullptr;       // weights are sigmoids of the scores and are not normalised
+  const float pb = sig ? mod.pb[h] : 0.f;
+  if (sig) m_run = 0.f;
+  const int kept = keep_tiles(mod.keep, CHUNK), lo_chunk = lo / CHUNK;
 
-  for (int base = (lo / CHUNK) * CHUNK; base <= pos; base += CHUNK) {
+  for (int c_i = first_tile(lo_chunk, kept); c_i * CHUNK <= pos; c_i = next_tile(c_i, lo_chunk, kept)) {
+    const int base = c_i * CHUNK;
     const int j = base + tid;
-    const bool valid = j >= lo && j <= pos;
+    const bool valid = sees(j, pos, lo, mod.keep);
     float sc = -INFINITY;
     int64_t off = 0;
     if (valid) {
@@ -60,9 +65,9 @@ __global__ __launch_bounds__(CHUNK) void attention_generic_kernel(
     }
     head_off[tid] = off;
     row_in_page[tid] = j % page_size;
-    const float m_chunk = block_max(sc, red);
+    const float m_chunk = sig ? 0.f : block_max(sc, red);
     const float m_new = fmaxf(m_run, m_chunk);
-    const float p = valid ? expf(sc - m_new) : 0.f;
+    const float p = valid ? (sig ? sigmoid_weight(sc + pb) : expf(sc - m_new)) : 0.f;
     ps[tid] = p;
     const float l_chunk = block_sum(p, red);   // has the barriers that publish ps and the offsets
     const float alpha = m_run == -INFINITY ? 0.f : expf(m_run - m_new);
@@ -84,13 +89,19 @@ __global__ __launch_bounds__(CHUNK) void attention_generic_kernel(
     }
     __syncthreads();
   }
-  const float inv = 1.0f / l_run;
+  const float inv = sig ? 1.0f : 1.0f / l_run;
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
     const int d = tid + c * CHUNK;
     if (d < hd) out[((size_t)t * nh + h) * hd + d] = from_f32<act_t>(acc[c] * inv);
   }
 }
+
+TQ_API int tq_attention_generic_sig(const void* q, const void* k_pool, const void* v_pool, const int* positions,
+                                    const int* seq_of_token, const int* block_table, int bt_stride, int page_size,
+                                    int64_t page_stride, int T, int nh, int nkv, int hd, int window, float scale,
+                                    float softcap, const float* r1, const float* r2, int chunk, const float* sink,
+                                    const float* pb, int keep, void* out, hipStream_t st);
 
 // softcap, r1, r2, chunk, sink: what happens to a score before the softmax and the chunks of positions, see score_mod.h
 // (0, null, null, 0, null: nothing).
@@ -99,9 +110,20 @@ TQ_API int tq_attention_generic_mod(const void* q, const void* k_pool, const voi
                                     int64_t page_stride, int T, int nh, int nkv, int hd, int window, float scale,
                                     float softcap, const float* r1, const float* r2, int chunk, const float* sink,
                                     void* out, hipStream_t st) {
+  return tq_attention_generic_sig(q, k_pool, v_pool, positions, seq_of_token, block_table, bt_stride, page_size,
+                                  page_stride, T, nh, nkv, hd, window, scale, softcap, r1, r2, chunk, sink, nullptr, 0,
+                                  out, st);
+}
+
+// pb, keep: sigmoid weights with a bias per head, and first positions that stay visible (score_mod.h; null, 0: neither).
+TQ_API int tq_attention_generic_sig(const void* q, const void* k_pool, const void* v_pool, const int* positions,
+                                    const int* seq_of_token, const int* block_table, int bt_stride, int page_size,
+                                    int64_t page_stride, int T, int nh, int nkv, int hd, int window, float scale,
+                                    float softcap, const float* r1, const float* r2, int chunk, const float* sink,
+                                    const float* pb, int keep, void* out, hipStream_t st) {
   if (T <= 0) return 0;
-  if ((r1 == nullptr) != (r2 == nullptr) || chunk < 0 || softcap < 0.f) return TQ_ERR_BAD_ARG;
-  const ScoreMod mod{softcap, r1, r2, chunk, sink};
+  if ((r1 == nullptr) != (r2 == nullptr) || chunk < 0 || softcap < 0.f || keep < 0 || (pb && sink)) return TQ_ERR_BAD_ARG;
+  const ScoreMod mod{softcap, r1, r2, chunk, sink, pb, keep};
   if (hd > 4 * CHUNK || nkv <= 0 || nh % nkv != 0) return TQ_ERR_UNSUPPORTED;
   if (nh > 65535) return TQ_ERR_UNSUPPORTED;
   const size_t shmem = (size_t)(hd + CHUNK + 4) * sizeof(float) + CHUNK * (sizeof(int64_t) + sizeof(int));

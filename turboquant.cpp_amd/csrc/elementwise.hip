@@ -148,7 +148,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const float* __restric
           f32x4 t[4];
 #pragma unroll
           for (int u = 0; u < 4; ++u)
-            if (j + u < topk) t[u] = load4f(y + (size_t)slot[j + u] * H + i);
+            if (j + u < topk) t[u] = slot[j + u] < 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : load4f(y + (size_t)slot[j + u] * H + i);
 #pragma unroll
           for (int u = 0; u < 4; ++u)
             if (j + u < topk) acc += wgt[j + u] * t[u];
@@ -190,7 +190,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const float* __restric
       float a = xr[i];
       if (y) {
         float acc = 0.f;
-        for (int j = 0; j < topk; ++j) acc += wgt[j] * y[(size_t)slot[j] * H + i];
+        for (int j = 0; j < topk; ++j) acc += slot[j] < 0 ? 0.f : wgt[j] * y[(size_t)slot[j] * H + i];
         if (S > 0) {
           float sh = 0.f;
           for (int s = 0; s < S; ++s) sh += dr[s * delta_stride + i];
@@ -833,7 +833,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
   const float g = gate ? gate[t] : 1.0f;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     float acc = 0.f;
-    for (int j = 0; j < topk; ++j) acc += wgt[j] * y[(size_t)slot[j] * H + i];
+    for (int j = 0; j < topk; ++j) acc += slot[j] < 0 ? 0.f : wgt[j] * y[(size_t)slot[j] * H + i];
     if (shared) {
       float sh = 0.f;
       for (int s = 0; s < S; ++s) sh += shared[s * shared_stride + (size_t)t * H + i];
@@ -920,6 +920,7 @@ __global__ void add_normed_rmsnorm_kernel(float* __restrict__ x, const float* __
     for (int u = 0; u < N; ++u) d[u] = 0.f;
     if (y) {
       for (int j = 0; j < topk; ++j) {
+        if (slot[j] < 0) continue;        // a pair without a row (an expert that is the identity: its share rides in `delta`)
         const float* yr = y + (size_t)slot[j] * H + i;
         if constexpr (VEC) {
           const f32x4 t = load4f(yr);
@@ -1013,6 +1014,93 @@ TQ_API int tq_add_normed_rmsnorm(float* x, const float* delta, int S, int64_t de
                          (size_t)delta_stride, y, pair_slot, weights, topk, gate, (const W*)wd, eps_d, (const W*)w, eps,
                          rows, (act_t*)out, out32, H);
     }
+  });
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- token shift
+// What a mixer reads where every token is blended with the token before it: out[t] = x[t] + (x[t-1] - x[t]) * w, x[t-1]
+// being the sequence's row before, as it was before any blending: the step's own row t - 1, or for the first token that
+// a sequence brings the row that its slot keeps from the step before (zeros for a new sequence).  Afterwards the slot
+// keeps the last row that the sequence brought.  The workgroup of a run's first token reads the slot's row and is the
+// one that writes it, each thread its own elements, so no other workgroup touches it in between.
+template <class W>
+__global__ __launch_bounds__(256) void token_shift_kernel(const float* __restrict__ x, const W* __restrict__ w,
+                                                          float* __restrict__ state, const int* __restrict__ cu_seqlens,
+                                                          const int* __restrict__ slots, int B, act_t* __restrict__ out, int H) {
+  const int t = blockIdx.x;
+  // the run that holds token t: the last one that starts at or before it
+  int lo = 0, hi = B - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) / 2;
+    if (cu_seqlens[mid] <= t) lo = mid; else hi = mid - 1;
+  }
+  const int first = cu_seqlens[lo], last = cu_seqlens[lo + 1] - 1;
+  const float* xr = x + (size_t)t * H;
+  if (t != first) {
+    const float* xp = xr - H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) out[(size_t)t * H + i] = from_f32<act_t>(xr[i] + (xp[i] - xr[i]) * to_f32(w[i]));
+    return;
+  }
+  float* sr = state + (size_t)slots[lo] * H;
+  const float* xl = x + (size_t)last * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float before = sr[i];
+    out[(size_t)t * H + i] = from_f32<act_t>(xr[i] + (before - xr[i]) * to_f32(w[i]));
+    sr[i] = xl[i];
+  }
+}
+
+// x float [T][H]; w [H]; state float [slots][H]; cu_seqlens [B + 1], slots [B]: the step's runs; out [T][H] in the
+// activation type.
+TQ_API int tq_token_shift(const float* x, const void* w, int wtype, float* state, const int* cu_seqlens, const int* slots,
+                          int B, void* out, int T, int H, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (B <= 0 || H <= 0) return TQ_ERR_BAD_ARG;
+  TQ_DISPATCH_W(wtype, {
+    hipLaunchKernelGGL(token_shift_kernel<W>, dim3(T), dim3(256), 0, st, x, (const W*)w, state, cu_seqlens, slots, B,
+                       (act_t*)out, H);
+  });
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- unit values, mixed with another layer's
+// Every value head of the float rows v [T][.. heads * hd ..] (row stride ld, head stride hd, a head's first vd numbers
+// its values) is divided by its root mean square over vd (eps inside the root, no weights; eps 0: left as it is), in place; with `first`
+// (another layer's rows of values, laid out alike with its own strides, already so normed) it then becomes
+// (1 - lambda) v + lambda first, lambda read from the device.  A wave takes a head of a token.
+template <class W>
+__global__ __launch_bounds__(256) void value_norm_mix_kernel(float* __restrict__ v, int64_t ld, int hd, int vd, int heads,
+                                                             float eps, const float* __restrict__ first, int64_t ld_first,
+                                                             int hd_first, const W* __restrict__ lambda, int T) {
+  const int wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
+  const int64_t item = (int64_t)blockIdx.x * (blockDim.x / TQ_WAVE) + wave;
+  if (item >= (int64_t)T * heads) return;
+  const int t = (int)(item / heads), h = (int)(item % heads);
+  float* row = v + (size_t)t * ld + (size_t)h * hd;
+  float ss = 0.f;
+  for (int i = lane; i < vd; i += TQ_WAVE) ss += row[i] * row[i];
+  ss = wave_sum(ss);
+  const float r = eps > 0.f ? 1.0f / sqrtf(ss / (float)vd + eps) : 1.0f;      // eps 0: the values are mixed as they are
+  const float lam = first ? to_f32(lambda[0]) : 0.f;
+  const float* fr = first ? first + (size_t)t * ld_first + (size_t)h * hd_first : nullptr;
+  for (int i = lane; i < vd; i += TQ_WAVE) {
+    float a = row[i] * r;
+    if (first) a = (1.0f - lam) * a + lam * fr[i];
+    row[i] = a;
+  }
+}
+
+TQ_API int tq_value_norm_mix(float* v, int64_t ld, int hd, int vd, int heads, float eps, const float* first,
+                             int64_t ld_first, int hd_first, const void* lambda, int wtype, int T, hipStream_t st) {
+  if (T <= 0 || heads <= 0) return 0;
+  if (vd < 1 || vd > hd || (first && (!lambda || vd > hd_first))) return TQ_ERR_BAD_ARG;
+  const int64_t items = (int64_t)T * heads;
+  TQ_DISPATCH_W(first ? wtype : TQ_F32, {
+    hipLaunchKernelGGL(value_norm_mix_kernel<W>, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, st, v, ld, hd, vd, heads, eps,
+                       first, ld_first, hd_first, (const W*)lambda, T);
   });
   TQ_LAUNCH_CHECK();
   return 0;

@@ -147,7 +147,8 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float* __restr
 // others are left out.
 __device__ __forceinline__ void select_token(const float* __restrict__ src, int rows, int E, int topk, int renorm,
                                              int groups, int keep, float* lg, int* __restrict__ ids, int* ids2,
-                                             float* __restrict__ weights, float* __restrict__ shared_gate) {
+                                             float* __restrict__ weights, float* __restrict__ shared_gate,
+                                             const float* __restrict__ correction = nullptr, int n_real = 1 << 30) {
   const int lane = threadIdx.x % TQ_WAVE;
   for (int e = lane; e < E; e += TQ_WAVE) lg[e] = src[e];
   if (rows > E && lane == 0) shared_gate[0] = 1.0f / (1.0f + expf(-src[E]));
@@ -160,6 +161,11 @@ __device__ __forceinline__ void select_token(const float* __restrict__ src, int 
     float d = 0.f;
     for (int e = lane; e < E; e += TQ_WAVE) d += expf(lg[e] - mx);
     denom = wave_sum(d);
+  }
+  if (correction) {
+    // the choice is by the softmax score plus a number per expert; the weights are the scores without it
+    for (int e = lane; e < E; e += TQ_WAVE) lg[e] = expf(lg[e] - mx) * (1.0f / denom) + correction[e];
+    __builtin_amdgcn_wave_barrier();
   }
   if (groups > 1 && keep < groups) {
     const int per = E / groups;
@@ -203,6 +209,7 @@ __device__ __forceinline__ void select_token(const float* __restrict__ src, int 
     __builtin_amdgcn_wave_barrier();
   }
   float sel = 0.f;    // lane k keeps the k-th selected logit
+  int sel_id = -1;    // and its expert
   for (int k = 0; k < topk; ++k) {
     float bv = -INFINITY;
     int bi = -1;
@@ -223,7 +230,10 @@ __device__ __forceinline__ void select_token(const float* __restrict__ src, int 
       }
     }
     if (bi < 0) bi = 0;   // only if every logit is NaN
-    if (lane == k) sel = bv;
+    if (lane == k) {
+      sel = correction ? src[bi] : bv;
+      sel_id = bi;
+    }
     if (lane == 0) {
       ids[k] = bi;
       if (ids2) ids2[k] = bi;
@@ -237,20 +247,26 @@ __device__ __forceinline__ void select_token(const float* __restrict__ src, int 
     const float s = wave_sum(p);
     if (lane < topk) weights[lane] = s > 0.f ? p * (1.0f / s) : 0.f;
   } else {
-    if (lane < topk) weights[lane] = expf(sel - mx) * (1.0f / denom);
+    const float wgt = lane < topk ? expf(sel - mx) * (1.0f / denom) : 0.f;
+    if (lane < topk) weights[lane] = wgt;
+    if (n_real < E) {     // experts from n_real on are the identity: the sum of their weights multiplies the token's own row
+      const float idw = wave_sum(sel_id >= n_real ? wgt : 0.f);
+      if (lane == 0) shared_gate[0] = idw;
+    }
   }
 }
 
 __global__ __launch_bounds__(256) void router_select_kernel(const float* __restrict__ logits, int rows, int E,
                                                             int topk, int renorm, int groups, int keep,
                                                             int* __restrict__ ids, float* __restrict__ weights,
-                                                            float* __restrict__ shared_gate, int T) {
+                                                            float* __restrict__ shared_gate, int T,
+                                                            const float* __restrict__ correction, int n_real) {
   extern __shared__ float sm[];      // [4][E]
   const int wave = threadIdx.x / TQ_WAVE;
   const int t = blockIdx.x * 4 + wave;
   if (t >= T) return;
   select_token(logits + (size_t)t * rows, rows, E, topk, renorm, groups, keep, sm + wave * E, ids + (size_t)t * topk, nullptr,
-               weights + (size_t)t * topk, shared_gate + t);
+               weights + (size_t)t * topk, shared_gate + t, correction, n_real);
 }
 
 static int launch_router_logits(const float* x, const void* wr, const void* shared_w, int wtype, int E,
@@ -302,9 +318,9 @@ static int groups_ok(int E, int topk, int groups, int keep) {
 }
 
 // bias (null, or float [E]): added to the experts' logits before the choice.
-TQ_API int tq_router_topk_biased(const float* x, const void* wr, const void* shared_w, const float* bias, int wtype, int E,
-                                 int topk, int renorm, int groups, int keep, int* ids, float* weights, float* shared_gate,
-                                 float* logits, int T, int H, hipStream_t st) {
+static int router_topk_impl(const float* x, const void* wr, const void* shared_w, const float* bias, int wtype, int E,
+                            int topk, int renorm, int groups, int keep, int* ids, float* weights, float* shared_gate,
+                            float* logits, int T, int H, hipStream_t st, const float* correction, int n_real) {
   if (T <= 0) return 0;
   if (topk < 1 || topk > 64 || topk > E || E > 8192) return TQ_ERR_UNSUPPORTED;
   if (!groups_ok(E, topk, groups, keep)) return TQ_ERR_BAD_ARG;
@@ -312,9 +328,16 @@ TQ_API int tq_router_topk_biased(const float* x, const void* wr, const void* sha
   if (rc) return rc;
   const int rows = E + (shared_w ? 1 : 0);
   hipLaunchKernelGGL(router_select_kernel, dim3((T + 3) / 4), dim3(256), (size_t)4 * E * sizeof(float), st, logits,
-                     rows, E, topk, renorm, groups, keep, ids, weights, shared_gate, T);
+                     rows, E, topk, renorm, groups, keep, ids, weights, shared_gate, T, correction, n_real);
   TQ_LAUNCH_CHECK();
   return 0;
+}
+
+TQ_API int tq_router_topk_biased(const float* x, const void* wr, const void* shared_w, const float* bias, int wtype, int E,
+                                 int topk, int renorm, int groups, int keep, int* ids, float* weights, float* shared_gate,
+                                 float* logits, int T, int H, hipStream_t st) {
+  return router_topk_impl(x, wr, shared_w, bias, wtype, E, topk, renorm, groups, keep, ids, weights, shared_gate, logits, T, H,
+                          st, nullptr, E);
 }
 
 TQ_API int tq_router_topk_grouped(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk,
@@ -426,7 +449,9 @@ __device__ __forceinline__ void scan_starts(int* starts, int E, int unit, int ca
 template <int NW>
 __device__ __forceinline__ void align_pairs(const int* ids, int n_pairs, int E, int topk, int unit, int cap,
                                             int* __restrict__ sorted_token, int* __restrict__ pair_slot,
-                                            int* __restrict__ tile_expert, int* __restrict__ n_tiles, int* cnt) {
+                                            int* __restrict__ tile_expert, int* __restrict__ n_tiles, int* cnt,
+                                            int n_real = 1 << 30) {
+  // (experts from n_real on have no matrices: their pairs get no rows, pair_slot -1, and they no tiles)
   int* starts = cnt + NW * E;
   const int wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
   for (int i = threadIdx.x; i < cap; i += blockDim.x) sorted_token[i] = -1;
@@ -449,13 +474,15 @@ __device__ __forceinline__ void align_pairs(const int* ids, int n_pairs, int E, 
       cnt[w * E + e] = total;
       total += c;
     }
-    starts[e] = (total + unit - 1) / unit * unit;
+    starts[e] = e < n_real ? (total + unit - 1) / unit * unit : 0;
   }
   __syncthreads();
   if (wave == 0) scan_starts(starts, E, unit, cap, tile_expert, n_tiles);
   __syncthreads();
   if (one_batch) {
-    if (my_e >= 0) {
+    if (my_e >= n_real) {
+      pair_slot[threadIdx.x] = -1;
+    } else if (my_e >= 0) {
       const int i = threadIdx.x;
       const int r = starts[my_e] + cnt[wave * E + my_e] + my_rank;
       pair_slot[i] = r;
@@ -465,6 +492,10 @@ __device__ __forceinline__ void align_pairs(const int* ids, int n_pairs, int E, 
   }
   for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) {
     const int e = ids[i], w = i / per;
+    if (e >= n_real) {
+      pair_slot[i] = -1;
+      continue;
+    }
     const int r = starts[e] + cnt[w * E + e] + pair_slot[i];
     pair_slot[i] = r;
     sorted_token[r] = i / topk;
@@ -476,9 +507,9 @@ __global__ __launch_bounds__(64 * AW) void moe_align_kernel(const int* __restric
                                                             int* __restrict__ sorted_token,
                                                             int* __restrict__ pair_slot,
                                                             int* __restrict__ tile_expert,
-                                                            int* __restrict__ n_tiles) {
+                                                            int* __restrict__ n_tiles, int n_real) {
   extern __shared__ int cnt[];
-  align_pairs<AW>(ids, n_pairs, E, topk, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles, cnt);
+  align_pairs<AW>(ids, n_pairs, E, topk, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles, cnt, n_real);
 }
 
 // The same order by several workgroups, for steps of many tokens (one workgroup's waves go through 32,768 pairs in
@@ -507,7 +538,8 @@ __global__ __launch_bounds__(64 * AW) void align_count_kernel(const int* __restr
 }
 
 __global__ __launch_bounds__(64 * AW) void align_scan_kernel(int* __restrict__ table, int V, int E, int unit, int cap,
-                                                             int* __restrict__ tile_expert, int* __restrict__ n_tiles) {
+                                                             int* __restrict__ tile_expert, int* __restrict__ n_tiles,
+                                                             int n_real) {
   extern __shared__ int sm_a[];        // [chunks][E] sums of AC waves' counts, then E starts
   const int chunks = (V + AC - 1) / AC;
   int* starts = sm_a + chunks * E;
@@ -527,7 +559,7 @@ __global__ __launch_bounds__(64 * AW) void align_scan_kernel(int* __restrict__ t
       sm_a[c * E + e] = total;
       total += t;
     }
-    starts[e] = (total + unit - 1) / unit * unit;
+    starts[e] = e < n_real ? (total + unit - 1) / unit * unit : 0;
   }
   __syncthreads();
   for (int idx = threadIdx.x; idx < chunks * E; idx += blockDim.x) {
@@ -551,7 +583,7 @@ __global__ __launch_bounds__(64 * AW) void align_scan_kernel(int* __restrict__ t
 __global__ __launch_bounds__(64 * AW) void align_place_kernel(const int* __restrict__ ids, int n_pairs, int E, int topk,
                                                               const int* __restrict__ table,
                                                               int* __restrict__ pair_slot,
-                                                              int* __restrict__ sorted_token) {
+                                                              int* __restrict__ sorted_token, int n_real) {
   extern __shared__ int sm_a[];        // [AW][E] first rows of this workgroup's waves within the experts, then E starts
   const int wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
   const int V = gridDim.x * AW, v = blockIdx.x * AW + wave;
@@ -573,7 +605,9 @@ __global__ __launch_bounds__(64 * AW) void align_place_kernel(const int* __restr
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int i = i0 + u * TQ_WAVE;
-      if (i < seg_end) {
+      if (i < seg_end && e[u] >= n_real) {
+        pair_slot[i] = -1;
+      } else if (i < seg_end) {
         const int r = starts[e[u]] + off[e[u]] + rk[u];
         pair_slot[i] = r;
         sorted_token[r] = i / topk;
@@ -597,7 +631,8 @@ static int align_workgroups(int n_pairs, int E, size_t table_ints) {
 }
 
 static int launch_align_multi(const int* ids, int n_pairs, int E, int topk, int unit, int cap, int* sorted_token,
-                              int* pair_slot, int* tile_expert, int* n_tiles, int* table, int g, hipStream_t st) {
+                              int* pair_slot, int* tile_expert, int* n_tiles, int* table, int g, hipStream_t st,
+                              int n_real = 1 << 30) {
   const int V = g * AW, chunks = (V + AC - 1) / AC;
   const size_t lds_count = (size_t)AW * E * sizeof(int), lds_scan = (size_t)(chunks + 1) * E * sizeof(int),
                lds_place = (size_t)(AW + 1) * E * sizeof(int);
@@ -610,9 +645,9 @@ static int launch_align_multi(const int* ids, int n_pairs, int E, int topk, int 
   hipLaunchKernelGGL(align_count_kernel, dim3(g), dim3(64 * AW), lds_count, st, ids, n_pairs, E, cap, sorted_token,
                      pair_slot, table);
   hipLaunchKernelGGL(align_scan_kernel, dim3(1), dim3(64 * AW), lds_scan, st, table, V, E, unit, cap, tile_expert,
-                     n_tiles);
+                     n_tiles, n_real);
   hipLaunchKernelGGL(align_place_kernel, dim3(g), dim3(64 * AW), lds_place, st, ids, n_pairs, E, topk, table, pair_slot,
-                     sorted_token);
+                     sorted_token, n_real);
   TQ_LAUNCH_CHECK();
   return 0;
 }
@@ -627,7 +662,8 @@ __global__ __launch_bounds__(64 * NW) void select_align_kernel(const float* __re
                                                                int cap, int* __restrict__ sorted_token,
                                                                int* __restrict__ pair_slot,
                                                                int* __restrict__ tile_expert,
-                                                               int* __restrict__ n_tiles) {
+                                                               int* __restrict__ n_tiles,
+                                                               const float* __restrict__ correction, int n_real) {
   extern __shared__ int sm_i[];       // (NW + 1) * E ints for the order, NW * topk ids, NW * E floats for the choice
   int* cnt = sm_i;
   int* ids_l = cnt + (NW + 1) * E;
@@ -635,15 +671,15 @@ __global__ __launch_bounds__(64 * NW) void select_align_kernel(const float* __re
   const int wave = threadIdx.x / TQ_WAVE;
   if (wave < T)
     select_token(logits + (size_t)wave * rows, rows, E, topk, renorm, groups, keep, lg + wave * E, ids + (size_t)wave * topk,
-                 ids_l + wave * topk, weights + (size_t)wave * topk, shared_gate + wave);
+                 ids_l + wave * topk, weights + (size_t)wave * topk, shared_gate + wave, correction, n_real);
   __syncthreads();
-  align_pairs<NW>(ids_l, T * topk, E, topk, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles, cnt);
+  align_pairs<NW>(ids_l, T * topk, E, topk, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles, cnt, n_real);
 }
 
 // cap: rows that sorted_token holds, a multiple of unit and at least n_pairs + min(E, n_pairs) * (unit - 1);
 // tile_expert holds 2 * cap / unit entries (row tiles, then items), n_tiles two.
-TQ_API int tq_moe_align(const int* ids, int n_pairs, int E, int topk, int unit, int cap, int* sorted_token,
-                        int* pair_slot, int* tile_expert, int* n_tiles, hipStream_t st) {
+static int moe_align_impl(const int* ids, int n_pairs, int E, int topk, int unit, int cap, int* sorted_token,
+                          int* pair_slot, int* tile_expert, int* n_tiles, hipStream_t st, int n_real) {
   if (n_pairs <= 0) return 0;
   if (unit < 1 || cap % unit != 0 || cap < n_pairs + (E < n_pairs ? E : n_pairs) * (unit - 1)) return TQ_ERR_BAD_ARG;
   const size_t shmem = (size_t)(AW + 1) * E * sizeof(int);
@@ -651,33 +687,38 @@ TQ_API int tq_moe_align(const int* ids, int n_pairs, int E, int topk, int unit, 
   if (shmem > 48 * 1024)
     (void)hipFuncSetAttribute((const void*)moe_align_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(64 * AW), shmem, st, ids, n_pairs, E, topk, unit, cap,
-                     sorted_token, pair_slot, tile_expert, n_tiles);
+                     sorted_token, pair_slot, tile_expert, n_tiles, n_real);
   TQ_LAUNCH_CHECK();
   return 0;
+}
+
+TQ_API int tq_moe_align(const int* ids, int n_pairs, int E, int topk, int unit, int cap, int* sorted_token,
+                        int* pair_slot, int* tile_expert, int* n_tiles, hipStream_t st) {
+  return moe_align_impl(ids, n_pairs, E, topk, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles, st, E);
 }
 
 // tq_router_topk followed by tq_moe_align; up to 16 tokens take two kernels instead of three, and from 8,192 pairs on
 // several workgroups order the pairs (the same order).  logits: scratch of T * (E + 1) floats (T * E without a shared
 // gate vector); what it holds afterwards means nothing.
 // groups, keep: the choice within the best `keep` of `groups` groups of experts (1, 1: among all).
-TQ_API int tq_route_biased(const float* x, const void* wr, const void* shared_w, const float* bias, int wtype, int E,
-                           int topk, int renorm, int groups, int keep, int* ids, float* weights, float* shared_gate,
-                           float* logits, int unit, int cap, int* sorted_token, int* pair_slot, int* tile_expert,
-                           int* n_tiles, int T, int H, hipStream_t st) {
+static int route_impl(const float* x, const void* wr, const void* shared_w, const float* bias, int wtype, int E,
+                      int topk, int renorm, int groups, int keep, int* ids, float* weights, float* shared_gate,
+                      float* logits, int unit, int cap, int* sorted_token, int* pair_slot, int* tile_expert,
+                      int* n_tiles, int T, int H, hipStream_t st, const float* correction, int n_real) {
   if (T <= 0) return 0;
   if (!groups_ok(E, topk, groups, keep)) return TQ_ERR_BAD_ARG;
   const size_t shmem = ((size_t)(AW + 1) * E + (size_t)AW * topk + (size_t)AW * E) * 4;
   if (T > AW || shmem > 64 * 1024) {
-    const int rc = tq_router_topk_biased(x, wr, shared_w, bias, wtype, E, topk, renorm, groups, keep, ids, weights,
-                                         shared_gate, logits, T, H, st);
+    const int rc = router_topk_impl(x, wr, shared_w, bias, wtype, E, topk, renorm, groups, keep, ids, weights,
+                                    shared_gate, logits, T, H, st, correction, n_real);
     if (rc) return rc;
     // once the experts are chosen the logits are done with: the order by several workgroups keeps its table there
     const int n = T * topk;
     const int g = align_workgroups(n, E, (size_t)T * (E + (shared_w ? 1 : 0)));
-    if (g == 0) return tq_moe_align(ids, n, E, topk, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles, st);
+    if (g == 0) return moe_align_impl(ids, n, E, topk, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles, st, n_real);
     if (unit < 1 || cap % unit != 0 || cap < n + (E < n ? E : n) * (unit - 1)) return TQ_ERR_BAD_ARG;
     return launch_align_multi(ids, n, E, topk, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles, (int*)logits, g,
-                              st);
+                              st, n_real);
   }
   if (topk < 1 || topk > 64 || topk > E || E > 8192) return TQ_ERR_UNSUPPORTED;
   const int n_pairs = T * topk;
@@ -687,16 +728,37 @@ TQ_API int tq_route_biased(const float* x, const void* wr, const void* shared_w,
   if (T == 1) {      // one wave: its barriers cost nothing
     const size_t shmem1 = ((size_t)2 * E + topk + E) * 4;
     hipLaunchKernelGGL(select_align_kernel<1>, dim3(1), dim3(64), shmem1, st, logits, E + (shared_w ? 1 : 0), E, topk,
-                       renorm, groups, keep, ids, weights, shared_gate, T, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles);
+                       renorm, groups, keep, ids, weights, shared_gate, T, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles,
+                       correction, n_real);
     TQ_LAUNCH_CHECK();
     return 0;
   }
   if (shmem > 48 * 1024)
     (void)hipFuncSetAttribute((const void*)select_align_kernel<AW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   hipLaunchKernelGGL(select_align_kernel<AW>, dim3(1), dim3(64 * AW), shmem, st, logits, E + (shared_w ? 1 : 0), E, topk,
-                     renorm, groups, keep, ids, weights, shared_gate, T, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles);
+                     renorm, groups, keep, ids, weights, shared_gate, T, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles,
+                       correction, n_real);
   TQ_LAUNCH_CHECK();
   return 0;
+}
+
+TQ_API int tq_route_biased(const float* x, const void* wr, const void* shared_w, const float* bias, int wtype, int E,
+                           int topk, int renorm, int groups, int keep, int* ids, float* weights, float* shared_gate,
+                           float* logits, int unit, int cap, int* sorted_token, int* pair_slot, int* tile_expert,
+                           int* n_tiles, int T, int H, hipStream_t st) {
+  return route_impl(x, wr, shared_w, bias, wtype, E, topk, renorm, groups, keep, ids, weights, shared_gate, logits, unit, cap,
+                    sorted_token, pair_slot, tile_expert, n_tiles, T, H, st, nullptr, E);
+}
+
+// A router whose softmax runs over all E rows, whose choice is by score + correction[e] and whose weights are the scores
+// themselves, not renormalised.  The rows from n_real on are experts without matrices (the identity): their pairs get
+// pair_slot -1 and no rows, and id_gate[t] (null if n_real == E) is the sum of the token's weights for them.
+TQ_API int tq_route_scored(const float* x, const void* wr, const float* correction, int wtype, int E, int n_real, int topk,
+                           int* ids, float* weights, float* id_gate, float* logits, int unit, int cap, int* sorted_token,
+                           int* pair_slot, int* tile_expert, int* n_tiles, int T, int H, hipStream_t st) {
+  if (n_real < 1 || n_real > E || (n_real < E && !id_gate) || !correction) return TQ_ERR_BAD_ARG;
+  return route_impl(x, wr, nullptr, nullptr, wtype, E, topk, 0, 1, 1, ids, weights, id_gate, logits, unit, cap, sorted_token,
+                    pair_slot, tile_expert, n_tiles, T, H, st, correction, n_real);
 }
 
 TQ_API int tq_route_grouped(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk, int renorm,

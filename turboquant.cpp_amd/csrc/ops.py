@@ -63,6 +63,14 @@ _SIGNATURES = {
                               _c_int, _c_f32, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "tq_attention_generic_mod": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_i64, _c_int, _c_int,
                                  _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr],
+    "tq_attention_generic_sig": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_i64, _c_int, _c_int,
+                                 _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr,
+                                 _c_ptr],
+    "tq_route_scored": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
+                        _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
+    "tq_token_shift": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr],
+    "tq_value_norm_mix": [_c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_f32, _c_ptr, _c_i64, _c_int, _c_ptr, _c_int, _c_int,
+                          _c_ptr],
     "tq_act_rows": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "tq_gate_rows": [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "tq_latent_norm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_f32, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_ptr],
@@ -128,6 +136,12 @@ _OPTIONAL = {
     "tq_attention_f32_mod": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
                              _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
                              _c_int, _c_int, _c_ptr],
+    "tq_attention_f32_sig": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
+                             _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr,
+                             _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "tq_attention_mfma_sig": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int,
+                              _c_int, _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr,
+                              _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr],
     "tq_attention_mfma_mod": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
                               _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
                               _c_int, _c_int, _c_ptr],
@@ -822,6 +836,18 @@ def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None
               "partial sums are for plain products into float32")
     lib = library(act)
     gate = _gate_code(k, activation)
+    if act_alone and (grouped or a_rows is not None):
+        # a product over experts whose result passes an activation: in the matrix-core product's own epilogue, else behind it
+        _need(w2 is None and not partial_sums and out_act, k, "an activation alone leaves its result in the activation type")
+        if _use_mfma(act, a, w, K) and (bias is None or bias.dtype in _WTYPE):
+            out = torch.empty((M, N), dtype=adt, device=a.device)
+            _run("gemm_mfma", lib.tq_gemm_mfma(_ptr(a), a.stride(0), _ptr(a_rows), int(gather), _ptr(w), None, gstride,
+                                               _ptr(tile_group), _ptr(n_tiles), _ptr(bias),
+                                               _WTYPE[bias.dtype] if bias is not None else 0, _ptr(out), N, 1, M, N, K,
+                                               tile_rows, 1, gate + 256, _stream()), "moe" if grouped else None)
+            return out
+        return act_rows(gemm(a, w, act, bias=bias, a_rows=a_rows, tile_group=tile_group, n_tiles=n_tiles, tile_rows=tile_rows,
+                             gather=gather), None, activation, act)
     if act_alone:
         _need(w2 is None and not partial_sums and not grouped and a_rows is None, k, "an activation alone is for plain products")
         if (dtype_name(act) == "bfloat16" and not (bias is None and _vendor_product(act, a, w, M, K))
@@ -926,7 +952,8 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
               scale: float, act, runs: dict | None = None, softcap: float | None = None,
               distance_bias: tuple[torch.Tensor, torch.Tensor] | None = None, chunk: int | None = None,
               sink: torch.Tensor | None = None, value_width: int | None = None,
-              head_gate: torch.Tensor | None = None) -> torch.Tensor:
+              head_gate: torch.Tensor | None = None, sigmoid_bias: torch.Tensor | None = None,
+              keep_first: int = 0) -> torch.Tensor:
     """Each token attends to its sequence's cached positions up to its own; returns [T, nh*hd].
 
     ``value_width``: a head's value rows hold zeros behind their first ``value_width`` numbers (keys wider than values, both
@@ -938,6 +965,9 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
     r1[h] ln(1 + r2[h] (i - j)) is taken off the score of query position i and key position j.  ``chunk`` n: position i
     sees j only if i // n == j // n, beside j <= i and the window.  ``sink`` float32 [nh]: the softmax's denominator of
     head h also holds exp(sink[h]), a score without key and value that is neither scaled nor capped and counts once.
+    ``sigmoid_bias`` float32 [nh]: no softmax; the weight of a visible key is sigmoid(score + sigmoid_bias[h]) and the
+    weights are not normalised over the keys.  ``keep_first`` n: the sequence's first n positions stay visible to every
+    later token, whatever the window.
 
     ``seq_of_token`` gives each token's row of ``block_table`` (its slot).  ``runs`` describes the same tokens
     as runs of consecutive positions, one per sequence, for the kernels that work on tiles of tokens:
@@ -972,9 +1002,15 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
         _check(r2, k, "r2", torch.float32, (num_heads,))
     if sink is not None:
         _check(sink, k, "sink", torch.float32, (num_heads,))
+    if sigmoid_bias is not None:
+        _check(sigmoid_bias, k, "sigmoid_bias", torch.float32, (num_heads,))
+        _need(sink is None, k, "sigmoid weights have no denominator for a sink to join")
+    _need(keep_first >= 0, k, "keep_first counts positions")
     mod = (cap, _ptr(r1), _ptr(r2), int(chunk or 0), _ptr(sink))
+    sig = (_ptr(sigmoid_bias), int(keep_first))
     if (runs is not None and dtype_name(act) == "bfloat16" and hasattr(lib, "tq_attention_mfma")
-            and head_dim % 16 == 0 and head_dim <= 512 and page_size % 64 == 0 and page_stride % 8 == 0 and scale > 0):
+            and head_dim % 16 == 0 and head_dim <= 512 and page_size % 64 == 0 and page_stride % 8 == 0 and scale > 0
+            and ((sigmoid_bias is None and keep_first == 0) or hasattr(lib, "tq_attention_mfma_sig"))):
         B = runs["slots"].numel()
         _check(runs["cu_seqlens"], k, "cu_seqlens", torch.int32, (B + 1,))
         _check(runs["slots"], k, "slots", torch.int32, (B,))
@@ -985,12 +1021,13 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
             _need(T == B, k, "decoding brings one token per sequence")
             partial = torch.empty((lib.tq_attention_decode_scratch(B, num_heads, head_dim, int(runs["max_end"])),),
                                   dtype=torch.float32, device=q.device)
-        _run("attention_mfma", lib.tq_attention_mfma_ex(
+        plain = sigmoid_bias is None and keep_first == 0
+        _run("attention_mfma", (lib.tq_attention_mfma_ex if plain else lib.tq_attention_mfma_sig)(
             _ptr(q), k_pages.data_ptr() + layer_offset * esz, v_pages.data_ptr() + layer_offset * esz,
             _ptr(block_table), block_table.shape[1], _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]), _ptr(runs["start"]),
             page_size, page_stride, B, num_heads, num_kv_heads, head_dim, int(window or 0), float(scale), *mod, _ptr(out),
             _ptr(partial), int(bool(runs["decode"])), int(runs["max_new"]), int(runs["max_end"]), int(value_width or 0),
-            _ptr(head_gate), head_gate.stride(0) if head_gate is not None else 0, _stream()))
+            _ptr(head_gate), head_gate.stride(0) if head_gate is not None else 0, *(() if plain else sig), _stream()))
         return out
     if (runs is not None and dtype_name(act) == "float32" and hasattr(lib, "tq_attention_f32") and head_dim % 4 == 0
             and head_dim <= 256 and page_size % 64 == 0 and page_stride % 4 == 0 and layer_offset % 4 == 0):
@@ -1004,17 +1041,17 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
             _need(T == B, k, "decoding brings one token per sequence")
             partial = torch.empty((lib.tq_attention_f32_scratch(B, num_heads, head_dim, int(runs["max_end"])),),
                                   dtype=torch.float32, device=q.device)
-        _run("attention_f32", lib.tq_attention_f32_mod(
+        _run("attention_f32", lib.tq_attention_f32_sig(
             _ptr(q), k_pages.data_ptr() + layer_offset * esz, v_pages.data_ptr() + layer_offset * esz,
             _ptr(block_table), block_table.shape[1], _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]), _ptr(runs["start"]),
-            page_size, page_stride, B, num_heads, num_kv_heads, head_dim, int(window or 0), float(scale), *mod, _ptr(out),
+            page_size, page_stride, B, num_heads, num_kv_heads, head_dim, int(window or 0), float(scale), *mod, *sig, _ptr(out),
             _ptr(partial), int(bool(runs["decode"])), int(runs["max_new"]), int(runs["max_end"]), _stream()))
         return out if head_gate is None else gate_heads(out, head_gate, num_heads, "sigmoid", act)
-    _run(k, lib.tq_attention_generic_mod(_ptr(q), k_pages.data_ptr() + layer_offset * esz,
+    _run(k, lib.tq_attention_generic_sig(_ptr(q), k_pages.data_ptr() + layer_offset * esz,
                                          v_pages.data_ptr() + layer_offset * esz, _ptr(positions),
                                          _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], page_size,
                                          page_stride, T, num_heads, num_kv_heads, head_dim, int(window or 0),
-                                         float(scale), *mod, _ptr(out), _stream()))
+                                         float(scale), *mod, *sig, _ptr(out), _stream()))
     return out if head_gate is None else gate_heads(out, head_gate, num_heads, "sigmoid", act)
 
 
@@ -1080,12 +1117,31 @@ def _align_outputs(T: int, topk: int, num_experts: int, unit: int, dev):
 
 
 def route(x32: torch.Tensor, router: torch.Tensor, shared_scale: torch.Tensor | None, top_k: int, renormalize: bool,
-          unit: int, act, groups: tuple[int, int] | None = None, bias: torch.Tensor | None = None):
+          unit: int, act, groups: tuple[int, int] | None = None, bias: torch.Tensor | None = None,
+          correction: torch.Tensor | None = None, identity: int = 0):
     """``router_topk`` followed by ``moe_align`` in one call: (ids, weights, gate, sorted_token, pair_slot,
-    tile_expert, n_tiles), with the same results; a handful of tokens takes one kernel less."""
+    tile_expert, n_tiles), with the same results; a handful of tokens takes one kernel less.
+
+    ``correction`` float32 [E] (with ``renormalize`` false and neither groups, bias nor shared gate): the softmax runs over
+    all E rows of the router, the choice is by score + correction and the weights are the scores themselves.  ``identity`` n
+    (with ``correction``): the router's last n rows are experts without matrices whose output is their input; their pairs
+    get ``pair_slot`` -1 and no rows in the order, and ``gate`` [T] is the sum of each token's weights for them."""
     k = "route"
     T, H, E, ids, weights, gate, logits = _router_outputs(k, x32, router, shared_scale, top_k)
     _need(unit in (16, 32, 64, 128, 256), k, "unit must be 16, 32, 64, 128 or 256")
+    if correction is not None:
+        _need(not renormalize and groups is None and bias is None and shared_scale is None and 0 <= identity < E, k,
+              "a choice by corrected scores goes with plain softmax weights over all experts, of which some are real")
+        _check(correction, k, "correction", torch.float32, (E,))
+        if identity:
+            gate = torch.empty((T,), dtype=torch.float32, device=x32.device)
+        cap, sorted_token, pair_slot, tile_expert, n_tiles = _align_outputs(T, top_k, E, unit, x32.device)
+        _run(k, library(act).tq_route_scored(_ptr(x32), _ptr(router), _ptr(correction), _WTYPE[router.dtype], E, E - identity,
+                                             top_k, _ptr(ids), _ptr(weights), _ptr(gate), _ptr(logits), unit, cap,
+                                             _ptr(sorted_token), _ptr(pair_slot), _ptr(tile_expert), _ptr(n_tiles), T, H,
+                                             _stream()))
+        return ids, weights, gate, sorted_token, pair_slot, tile_expert, n_tiles
+    _need(identity == 0, k, "experts that are the identity come with a choice by corrected scores")
     count, keep = _expert_groups(k, E, top_k, groups)
     if bias is not None:
         _check(bias, k, "bias", torch.float32, (E,))
@@ -1385,6 +1441,52 @@ def gate_rows(o: torch.Tensor, gate: torch.Tensor, activation: str, act) -> torc
           and gate.stride(1) == 1, k, lambda: f"gate must be float32 [{M}, {N}] on the GPU with unit stride along its rows")
     _run(k, library(act).tq_gate_rows(_ptr(o), _ptr(gate), gate.stride(0), _ptr(o), M, N, _gate_code(k, activation), _stream()))
     return o
+
+
+def token_shift(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, runs: dict, act) -> torch.Tensor:
+    """out[t] = x[t] + (x[t-1] - x[t]) * weight in the activation type, x[t-1] being the row of the sequence's token before:
+    the step's own row, or for a run's first token the row that ``state`` [slots, H] keeps for the sequence's slot (zeros
+    for a new sequence); afterwards the slot keeps the run's last row of ``x``.  ``runs`` as for ``attention``."""
+    k = "token_shift"
+    _check(x, k, "x", torch.float32)
+    _need(x.dim() == 2, k, "x must be [T, H]")
+    T, H = x.shape
+    _check(weight, k, "weight", tuple(_WTYPE), (H,))
+    _check(state, k, "state", torch.float32)
+    _need(state.dim() == 2 and state.shape[1] == H, k, lambda: f"state must be [slots, {H}]")
+    B = runs["slots"].numel()
+    _check(runs["cu_seqlens"], k, "cu_seqlens", torch.int32, (B + 1,))
+    _check(runs["slots"], k, "slots", torch.int32, (B,))
+    out = torch.empty((T, H), dtype=ACT_DTYPES[dtype_name(act)], device=x.device)
+    _run(k, library(act).tq_token_shift(_ptr(x), _ptr(weight), _WTYPE[weight.dtype], _ptr(state), _ptr(runs["cu_seqlens"]),
+                                        _ptr(runs["slots"]), B, _ptr(out), T, H, _stream()))
+    return out
+
+
+def value_norm_mix(v: torch.Tensor, num_heads: int, head_dim: int, value_dim: int, eps: float, act,
+                   first: torch.Tensor | None = None, first_head_dim: int | None = None,
+                   mix: torch.Tensor | None = None) -> torch.Tensor:
+    """Every value head of the float32 rows ``v`` [T, num_heads * head_dim] (columns of a wider tensor, a head's first
+    ``value_dim`` numbers its values) divided by its root mean square over them, in place, without weights; with ``first``
+    (another layer's values of the same tokens, so normed, laid out alike at ``first_head_dim`` a head) each then becomes
+    (1 - mix) v + mix first, ``mix`` a tensor of one number.  Returns ``v``."""
+    k = "value_norm_mix"
+    T = v.shape[0]
+    _need(v.is_cuda and v.dtype == torch.float32 and v.dim() == 2 and v.shape[1] == num_heads * head_dim and v.stride(1) == 1,
+          k, lambda: f"v must be float32 [T, {num_heads * head_dim}] on the GPU with unit stride along its rows")
+    _need(1 <= value_dim <= head_dim and eps >= 0, k, "the values lie within the head, and eps is positive (0: no norm)")
+    fhd = 0
+    if first is not None:
+        fhd = int(first_head_dim or head_dim)
+        _need(first.is_cuda and first.dtype == torch.float32 and first.dim() == 2 and first.shape[0] == T
+              and first.shape[1] == num_heads * fhd and first.stride(1) == 1 and value_dim <= fhd, k,
+              lambda: f"first must be float32 [{T}, {num_heads * fhd}] on the GPU with unit stride along its rows")
+        _check(mix, k, "mix", tuple(_WTYPE))
+        _need(mix.numel() == 1, k, "mix is one number")
+    _run(k, library(act).tq_value_norm_mix(_ptr(v), v.stride(0), head_dim, value_dim, num_heads, float(eps), _ptr(first),
+                                           first.stride(0) if first is not None else 0, fhd, _ptr(mix),
+                                           _WTYPE[mix.dtype] if first is not None else 0, T, _stream()))
+    return v
 
 
 def latent_norm(src: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, copies: int, width: int, act) -> None:

@@ -9,6 +9,11 @@
 //   sink           (per query head; null: none) the softmax's denominator also holds exp(sink[h]): a score that has no
 //                  key and no value, is not scaled, capped or biased, and counts once per query.  The kernels start
 //                  their running maximum at sink[h] with a denominator of 1 (the joins of decode steps add it once)
+//   pb             (per query head; null: none) no softmax: the weight of a visible key is sigmoid(score + pb[h]), and
+//                  the weights are not normalised over the keys.  The kernels keep their running maximum at 0, so that
+//                  nothing is ever rescaled, and leave the division by the sum out
+//   keep > 0       the first `keep` positions of a sequence stay visible to every later token, whatever the window:
+//                  position i sees j <= i if j >= reach_lo(i) or j < keep
 //
 // All of it in float, on both libraries.
 #pragma once
@@ -20,7 +25,22 @@ struct ScoreMod {
   const float* r2;
   int chunk;
   const float* sink;
+  const float* pb;
+  int keep;
 };
+
+// Tiles of `tile` positions that hold kept first positions, and the tile that follows tile t in a token's reach when
+// its window starts in tile `lo_tile`: the kept tiles come first, then the walk jumps to the window's first tile.
+__host__ __device__ __forceinline__ int keep_tiles(int keep, int tile) { return keep > 0 ? (keep + tile - 1) / tile : 0; }
+__host__ __device__ __forceinline__ int first_tile(int lo_tile, int kept) { return kept > 0 ? 0 : lo_tile; }
+__host__ __device__ __forceinline__ int next_tile(int t, int lo_tile, int kept) {
+  ++t;
+  return (t >= kept && t < lo_tile) ? lo_tile : t;
+}
+// whether a token at position p whose window starts at lo sees position j
+__host__ __device__ __forceinline__ bool sees(int j, int p, int lo, int keep) { return j <= p && (j >= lo || j < keep); }
+
+__device__ __forceinline__ float sigmoid_weight(float s) { return 1.0f / (1.0f + expf(-s)); }
 
 // the first position that a token at position p may see
 __host__ __device__ __forceinline__ int reach_lo(int p, int window, int chunk) {

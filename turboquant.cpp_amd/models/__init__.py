@@ -1,2 +1,2 @@
 """Architectures.  Importing this package registers every architecture it holds."""
-from . import beronex, felepel, qwen2_moe, taminex  # noqa: F401
+from . import beronex, bosalix, felepel, qwen2_moe, taminex  # noqa: F401

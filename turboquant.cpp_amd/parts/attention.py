@@ -21,6 +21,12 @@ the sigmoid of row h's product with the layer's input, before the output product
 value matrices: its schedule entry reads the cache of an earlier entry, with queries, window and everything else of its
 own); ``cache_window`` (what the cache keeps where that is more than the mixer's own window, because a later layer that
 reads this cache looks further back; None: everything).  A position part may scale its sines and cosines (``amplitude``).
+``value_norm_eps`` (every value head is divided by its root mean square over its width, no weights: the cache holds the
+values so normed); ``value_mix`` ("source": the layer leaves its values, as it caches them, for later layers of the same
+step; "mix": its values become (1 - mix) v + mix v_source, ``mix`` a learned number, before they are cached; both kinds
+carry the parameter, which a source does not use); ``sigmoid_bias`` (no softmax: the weight of a visible key is
+sigmoid(score + b_h), b a learned number per head, and the weights are not normalised over the keys); ``keep_first`` n
+(with a window: the sequence's first n positions stay visible to every later token and stay in the cache).
 With ``separate_qkv`` the heads are laid out at a kernel width that is the larger of key and value width rounded up to
 16: the added rows and columns of the matrices are zeros, which change no score and no output, and every head size
 then runs on the matrix-core kernels of both libraries.
@@ -44,7 +50,24 @@ class GroupedQueryAttention(Part):
                  scale: float | None = None, qk_norm_eps: float | None = None, score_cap: float | None = None,
                  distance_bias: bool = False, chunk: int | None = None, value_dim: int | None = None,
                  separate_qkv: bool = False, sink: bool = False, rotated_norm_eps: float | None = None,
-                 head_gate: bool = False, shares_kv: bool = False, cache_window: int | None | str = "own"):
+                 head_gate: bool = False, shares_kv: bool = False, cache_window: int | None | str = "own",
+                 value_norm_eps: float | None = None, value_mix: str | None = None, sigmoid_bias: bool = False,
+                 keep_first: int = 0):
+        if value_mix not in (None, "source", "mix"):
+            raise ValueError(f"value_mix is None, 'source' or 'mix', got {value_mix!r}")
+        if (value_norm_eps is not None or value_mix is not None or sigmoid_bias or keep_first) and not separate_qkv:
+            raise ValueError("normed or mixed values, sigmoid weights and kept first positions need separate_qkv")
+        if value_norm_eps is not None and not value_norm_eps > 0:
+            raise ValueError(f"value_norm_eps must be positive, got {value_norm_eps}")
+        if value_mix is not None and shares_kv:
+            raise ValueError("a layer that reads another layer's values has none of its own to mix")
+        if sigmoid_bias and sink:
+            raise ValueError("sigmoid weights have no denominator for a sink to join")
+        if keep_first < 0:
+            raise ValueError(f"keep_first counts positions, got {keep_first}")
+        self.value_norm_eps, self.value_mix, self.has_sigmoid_bias = value_norm_eps, value_mix, sigmoid_bias
+        self.keep_first = int(keep_first) if window is not None else 0      # without a window everything stays visible anyway
+        self.mix = self.score_bias = None
         if (head_gate or shares_kv) and not separate_qkv:
             raise ValueError("a gate per head and a cache shared with another layer need separate_qkv")
         if rotated_norm_eps is not None and not rotated_norm_eps > 0:
@@ -108,6 +131,10 @@ class GroupedQueryAttention(Part):
                 specs.update({"q_norm": ParamSpec((K,), role="scale"), "k_norm": ParamSpec((K,), role="scale")})
             if self.has_sink:
                 specs["sink"] = ParamSpec((H,), role="scale")
+            if self.has_sigmoid_bias:
+                specs["score_bias"] = ParamSpec((H,), role="scale")
+            if self.value_mix is not None:
+                specs["mix"] = ParamSpec((), role="scale")
             return specs
         rows = self.q_size + 2 * self.kv_size
         splits = (self.q_size, self.kv_size, self.kv_size)
@@ -133,6 +160,10 @@ class GroupedQueryAttention(Part):
             self.r1, self.r2 = self.r1.float().contiguous(), self.r2.float().contiguous()
         if self.has_sink:
             self.sink = self.sink.float().contiguous()
+        if self.has_sigmoid_bias:
+            self.score_bias = self.score_bias.float().contiguous()
+        if self.value_mix is not None:
+            self.mix = self.mix.reshape(1).contiguous()
         if not self.separate_qkv or self.qkv_weight is not None:
             return
         D = self.head_dim
@@ -171,7 +202,8 @@ class GroupedQueryAttention(Part):
         return {"position": self.position}
 
     def cache_need(self) -> CacheNeed:
-        return CacheNeed(self.num_kv_heads, self.head_dim, self.cache_window, chunk=self.chunk)
+        return CacheNeed(self.num_kv_heads, self.head_dim, self.cache_window, chunk=self.chunk,
+                         keep_first=self.keep_first if self.cache_window is not None else 0)
 
     def state_need(self):
         return None
@@ -203,12 +235,17 @@ class GroupedQueryAttention(Part):
             opts["chunk"] = self.chunk
         if self.has_sink:
             opts["sink"] = self.sink
+        if self.has_sigmoid_bias:
+            opts["sigmoid_bias"] = self.score_bias
+        if self.keep_first:
+            opts["keep_first"] = self.keep_first
         return opts
 
     def forward(self, normed, ctx, entry):
         b, kv = ctx.batch, ctx.kv(entry)
         amplitude = getattr(self.position, "amplitude", 1.0)
-        if self.rotated_norm_eps is not None or self.has_head_gate or self.shares_kv or amplitude != 1.0:
+        if (self.rotated_norm_eps is not None or self.has_head_gate or self.shares_kv or amplitude != 1.0
+                or self.value_norm_eps is not None or self.value_mix is not None):
             return self._forward_extended(normed, ctx, b, kv, amplitude)
         rope = (b.positions, b.slot_of_token, kv.table, self.position.table(ctx.device), self.position.pairing_code,
                 self.position.rotary_dim, kv.k_pages if kv.owns else None, kv.v_pages if kv.owns else None,
@@ -226,8 +263,8 @@ class GroupedQueryAttention(Part):
         return ops.gemm(o, self.out_weight, ctx.act, bias=self.out_bias, partial_sums=True)
 
     def _forward_extended(self, normed, ctx, b, kv, amplitude):
-        """The forms with a norm behind the rotation, scaled sines and cosines, a gate per head or another layer's keys
-        and values: one product of the layer's input (q | k | v | gate rows), the rotation with its norm and the cache
+        """The forms with a norm behind the rotation, scaled sines and cosines, a gate per head, another layer's keys
+        and values, or values that are normed or mixed with an earlier layer's: one product of the layer's input (q | k | v | gate rows), the rotation with its norm and the cache
         write in one launch, attention with the gate where it normalises its output, the output product."""
         if kv.owns == self.shares_kv:
             raise ValueError("an attention keeps a cache of its own exactly if it has keys and values of its own")
@@ -240,6 +277,15 @@ class GroupedQueryAttention(Part):
                 raise ValueError("the norm of the heads before the rotation does not go with a gate per head")
             ops.head_rmsnorm(qkv, self.q_norm, None if self.shares_kv else self.k_norm, self.qk_norm_eps, H, G, D, ctx.act,
                              norm_dim=self.key_dim)
+        if self.value_norm_eps is not None or self.value_mix is not None:
+            # the values as the cache will hold them: unit root mean square per head, then the blend with the values that
+            # the source layer left for this step's tokens
+            v = qkv[:, (H + G) * D:]
+            first, first_dim = b.scratch[("value_mix",)] if self.value_mix == "mix" else (None, None)
+            ops.value_norm_mix(v, G, D, self.value_dim, self.value_norm_eps or 0.0, ctx.act, first=first,
+                               first_head_dim=first_dim, mix=self.mix if first is not None else None)
+            if self.value_mix == "source":
+                b.scratch[("value_mix",)] = (v, D)
         q = ops.rope_kv_write(qkv, b.positions, b.slot_of_token, kv.table, self.position.table(ctx.device),
                               self.position.pairing_code, self.position.rotary_dim, kv.k_pages if kv.owns else None,
                               kv.v_pages if kv.owns else None, kv.layer_offset, kv.page_size, kv.page_stride, H, G, D, ctx.act,

@@ -16,6 +16,8 @@ Interfaces (``ctx`` is the :class:`~..engine.context.StepContext` of the running
             write the rows of the step's sequences through the slots on the device, which a decode step that is to
             be replayed must use).  ``cache_need()`` / ``state_need()`` say what storage each run wants.
 * ffn       ``forward(normed, normed32, ctx) -> delta``; ``wants_f32`` says whether it reads the float32 copy.
+* shift     ``forward(x, ctx, entry) -> h``: what a mixer reads of the float32 stream ``x`` where every token is blended with
+            the one before it; ``state_need()`` says what it keeps per sequence between steps.
 * position  ``table(device)``, ``pairing``, ``rotary_dim``: the rotation a mixer applies to queries and keys.
 * block     ``forward(x, pending, ctx, entry) -> pending``: the arrangement of norms, mixer and ffn around
             the residual stream.
@@ -48,12 +50,14 @@ class CacheNeed:
     """Keys and values per position: ``window`` None keeps all positions, else the last ``window``.
     ``head_dim`` is the width of a key row; ``value_dim`` that of a value row (None: the same; 0: no values are
     kept, one row per position and kv head only).  ``chunk`` n: a token sees only the positions of its own chunk of n
-    (counted from position 0), so what lies before the chunk of the next token need not be kept."""
+    (counted from position 0), so what lies before the chunk of the next token need not be kept.  ``keep_first`` n (with a
+    window): the sequence's first n positions stay in every later token's sight and are kept whatever the window."""
     num_kv_heads: int
     head_dim: int
     window: int | None = None
     value_dim: int | None = None
     chunk: int | None = None
+    keep_first: int = 0
 
     @property
     def value_width(self) -> int:
@@ -102,7 +106,7 @@ class Part:
 
 
 _REGISTRIES: dict[str, dict[str, Callable[..., Part]]] = {
-    "norm": {}, "mixer": {}, "ffn": {}, "position": {}, "block": {},
+    "norm": {}, "mixer": {}, "ffn": {}, "position": {}, "block": {}, "shift": {},
 }
 
 

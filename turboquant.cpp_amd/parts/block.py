@@ -94,34 +94,49 @@ class OutputNormBlock(Part):
     """A norm on every part's output only: ``x += norm_a(mixer(x)); x += norm_b(ffn(x))``.  The parts read the residual
     stream itself, un-normed, in the activation type; the feed-forward half is optional (``ffn`` and ``ffn_norm`` None: the
     layer is its mixer alone).  A part's output travels on wrapped with the weights of its norm (``ops.NormedDelta``), and
-    the kernel that sums it into the stream norms it in the same pass and hands the summed stream to the next part."""
+    the kernel that sums it into the stream norms it in the same pass and hands the summed stream to the next part.
+    ``mixer_shift`` (optional, a part of the "shift" registry): the mixer reads the stream blended token by token with the
+    row before (``parts/shift.py``) instead of the stream itself; the feed-forward still reads the stream.  What the shift
+    keeps per sequence is the layer's state, so it goes with mixers that keep none of their own.  A feed-forward that wants
+    its input in float32 as well (a router) is given the stream itself."""
     graph_safe = True
-    slots = {"mixer": "mixer", "mixer_norm": "norm", "ffn": "ffn", "ffn_norm": "norm"}
-    optional = ("ffn", "ffn_norm")
+    slots = {"mixer": "mixer", "mixer_norm": "norm", "ffn": "ffn", "ffn_norm": "norm", "mixer_shift": "shift"}
+    optional = ("ffn", "ffn_norm", "mixer_shift")
 
-    def __init__(self, mixer, mixer_norm, ffn=None, ffn_norm=None):
+    def __init__(self, mixer, mixer_norm, ffn=None, ffn_norm=None, mixer_shift=None):
         if (ffn is None) != (ffn_norm is None):
             raise ValueError("a layer has a feed-forward with its norm, or neither")
-        self.mixer, self.mixer_norm, self.ffn, self.ffn_norm = mixer, mixer_norm, ffn, ffn_norm
+        if mixer_shift is not None and mixer.state_need() is not None:
+            raise ValueError("a shifted input goes with a mixer that keeps no state of its own per sequence")
+        self.mixer, self.mixer_norm, self.ffn, self.ffn_norm, self.mixer_shift = mixer, mixer_norm, ffn, ffn_norm, mixer_shift
 
     def children(self):
-        parts = {"mixer": self.mixer, "mixer_norm": self.mixer_norm, "ffn": self.ffn, "ffn_norm": self.ffn_norm}
+        parts = {"mixer": self.mixer, "mixer_norm": self.mixer_norm, "ffn": self.ffn, "ffn_norm": self.ffn_norm,
+                 "mixer_shift": self.mixer_shift}
         return {k: v for k, v in parts.items() if v is not None}
 
     def cache_need(self):
         return self.mixer.cache_need()
 
     def state_need(self):
-        return self.mixer.state_need()
+        return self.mixer.state_need() if self.mixer_shift is None else self.mixer_shift.state_need()
 
     def forward(self, x, pending, ctx, entry):
         from ..csrc import ops
         if pending is not None and not isinstance(pending, ops.NormedDelta):     # a layer of another arrangement before this one
             ops.add_rmsnorm(x, pending, self.mixer_norm.weight, self.mixer_norm.eps, ctx.act, want_act=False)
             pending = None
-        h, _ = ops.add_rmsnorm(x, pending, None, 0.0, ctx.act, stream=True)
+        if self.mixer_shift is None:
+            h, _ = ops.add_rmsnorm(x, pending, None, 0.0, ctx.act, stream=True)
+        else:       # the sum alone, then the blend with the row before from the float32 stream
+            if pending is not None:
+                ops.add_rmsnorm(x, pending, None, 0.0, ctx.act)
+            h = self.mixer_shift.forward(x, ctx, entry)
         pending = ops.NormedDelta(self.mixer.forward(h, ctx, entry), self.mixer_norm.weight, self.mixer_norm.eps)
         if self.ffn is None:
             return pending
         h, _ = ops.add_rmsnorm(x, pending, None, 0.0, ctx.act, stream=True)
-        return ops.NormedDelta(self.ffn.forward(h, None, ctx), self.ffn_norm.weight, self.ffn_norm.eps)
+        # (a feed-forward that reads float32 rows reads the stream; what it hands on may name those rows, and the kernel
+        # that sums it into the stream reads a row whole before it writes that row)
+        return ops.NormedDelta(self.ffn.forward(h, x if getattr(self.ffn, "wants_f32", False) else None, ctx),
+                               self.ffn_norm.weight, self.ffn_norm.eps)

@@ -11,6 +11,10 @@ last.  ``renormalize`` false keeps the softmax over all experts un-normalised fo
 the reference's softmax over the chosen logits.  ``router_bias``: a number per expert is added to its logit before the
 choice.  ``pair_limit`` L: an expert is ``down(f(min(gate x, L)) * (clamp(up x, -L, L) + 1))``.  ``groups`` (count, keep): the experts form ``count`` equal groups of
 neighbours, a group's score is the largest score in it, and only experts of the ``keep`` best groups can be chosen.
+``gated`` false: an expert is ``down(f(up x))``, two matrices and no gate.  ``score_correction``: the softmax runs over all
+of the router's rows, the choice is by score plus a learned number per row, and the weights are the scores themselves,
+not renormalised.  ``identity`` n (with ``score_correction``): the router has n more rows than there are experts with
+matrices; a token that chooses one of them gets its own input back, times the weight.
 """
 from __future__ import annotations
 
@@ -87,14 +91,23 @@ class SparseMoE(Part):
 
     def __init__(self, hidden_size: int, num_experts: int, top_k: int, expert_size: int, shared_size: int = 0,
                  shared_gated: bool = True, renormalize: bool = False, activation: str = "silu",
-                 groups: tuple[int, int] | None = None, router_bias: bool = False, pair_limit: float | None = None):
+                 groups: tuple[int, int] | None = None, router_bias: bool = False, pair_limit: float | None = None,
+                 gated: bool = True, score_correction: bool = False, identity: int = 0):
+        if score_correction and (renormalize or groups is not None or router_bias or shared_size > 0):
+            raise ValueError("a choice by corrected scores goes with plain softmax weights over all rows, without groups, "
+                             "a router bias or a shared expert")
+        if identity < 0 or (identity and not score_correction):
+            raise ValueError("experts that are the identity come with a choice by corrected scores")
+        if not gated and pair_limit is not None:
+            raise ValueError("a limit is for gated pairs")
+        self.gated, self.score_correction, self.identity, self.correction = gated, score_correction, int(identity), None
         if pair_limit is not None and not pair_limit > 0:
             raise ValueError(f"pair_limit must be positive, got {pair_limit}")
         if (router_bias or pair_limit is not None) and shared_size > 0:
             raise ValueError("a router with a bias and experts with a limit come without a shared expert")
         self.has_router_bias, self.pair_limit, self.router_bias = router_bias, pair_limit, None
-        if not 1 <= top_k <= num_experts:
-            raise ValueError(f"top_k {top_k} must be within 1..num_experts {num_experts}")
+        if not 1 <= top_k <= num_experts + identity:
+            raise ValueError(f"top_k {top_k} must be within 1..{num_experts + identity}, the router's rows")
         if groups is not None:
             count, keep = groups
             if count < 1 or num_experts % count or not 1 <= keep <= count or top_k > keep * (num_experts // count):
@@ -112,9 +125,13 @@ class SparseMoE(Part):
 
     def param_specs(self):
         E, H, I, S = self.num_experts, self.hidden_size, self.expert_size, self.shared_size
-        specs = {"router": ParamSpec((E, H), role="router"),
+        specs = {"router": ParamSpec((E + self.identity, H), role="router"),
                  "expert_gate": ParamSpec((E, I, H)), "expert_up": ParamSpec((E, I, H)),
                  "expert_down": ParamSpec((E, H, I))}
+        if not self.gated:
+            del specs["expert_gate"]
+        if self.score_correction:
+            specs["correction"] = ParamSpec((E + self.identity,), role="bias")
         if self.has_router_bias:
             specs["router_bias"] = ParamSpec((E,), role="bias")
         if S > 0:
@@ -127,13 +144,15 @@ class SparseMoE(Part):
     def prepare(self, device, act):
         if self.has_router_bias:     # it enters float arithmetic only
             self.router_bias = self.router_bias.float().contiguous()
+        if self.score_correction:
+            self.correction = self.correction.float().contiguous()
         if self.shared_size > 0:     # as in the dense part; the experts' products never leave this library's kernels
             self.shared_gate, self.shared_up = ops.side_by_side(self.shared_gate, self.shared_up)
 
     def native(self):
         from ..csrc import host_api
         w = host_api.weight
-        if self.groups is not None or self.has_router_bias or self.pair_limit is not None:
+        if self.groups is not None or self.has_router_bias or self.pair_limit is not None or not self.gated or self.score_correction:
             return None                  # the executor chooses among all experts, by logits without a bias, for plain pairs
         return host_api.MoeFfnDesc(self.hidden_size, self.num_experts, self.top_k, self.expert_size, self.shared_size,
                                    int(self.renormalize), ops.GATES[self.activation], w(self.router),
@@ -142,8 +161,10 @@ class SparseMoE(Part):
 
     def forward(self, normed, normed32, ctx):
         T = normed.shape[0]
-        unit = ops.expert_tile_rows(T * self.top_k, self.num_experts, ctx.act, normed, self.expert_gate,
+        unit = ops.expert_tile_rows(T * self.top_k, self.num_experts, ctx.act, normed, self.expert_gate if self.gated else self.expert_up,
                                     **({} if self.expert_size % 8 == 0 else {"w_behind": self.expert_down}))
+        if self.score_correction or not self.gated:
+            return self._forward_scored(normed, normed32, ctx, unit)
         route = lambda: ops.route(normed32, self.router, self.shared_scale if self.shared_gated else None,
                                   self.top_k, self.renormalize, unit, ctx.act,
                                   **({} if self.groups is None else {"groups": self.groups}),
@@ -189,6 +210,25 @@ class SparseMoE(Part):
             ctx.join()
         # the weighted sum over the chosen experts and the shared expert is left to the next norm
         return ops.GatheredSum(y, pair_slot, weights, shared, gate)
+
+    def _forward_scored(self, normed, normed32, ctx, unit):
+        """Experts of two matrices, and routers that choose by corrected scores with experts that are the identity."""
+        T = normed.shape[0]
+        extra = {"correction": self.correction, "identity": self.identity} if self.score_correction else \
+            ({} if self.groups is None else {"groups": self.groups}) | ({} if self.router_bias is None else {"bias": self.router_bias})
+        _, weights, own, sorted_token, pair_slot, tile_expert, n_tiles = ops.route(
+            normed32, self.router, None, self.top_k, self.renormalize, unit, ctx.act, **extra)
+        rows = ops.expert_product_rows(unit, T * self.top_k, self.num_experts)
+        order = dict(a_rows=sorted_token, tile_group=tile_expert, n_tiles=n_tiles, tile_rows=rows)
+        if self.gated:
+            h = ops.gemm(normed, self.expert_gate, ctx.act, w2=self.expert_up, out_act=True, activation=self.activation,
+                         **order, **({} if self.pair_limit is None else {"pair_limit": self.pair_limit}))
+        else:
+            h = ops.gemm(normed, self.expert_up, ctx.act, out_act=True, activation=self.activation, act_alone=True, **order)
+        y = ops.gemm(h, self.expert_down, ctx.act, gather=False, **order)
+        # a token's weights for the experts that are the identity multiply its own float32 row, which rides where a shared
+        # expert's output would
+        return ops.GatheredSum(y, pair_slot, weights, normed32[None] if self.identity else None, own if self.identity else None)
 
     def _shared(self, normed, ctx):
         hs = ops.gemm(normed, self.shared_gate, ctx.act, w2=self.shared_up, out_act=True, activation=self.activation)

@@ -25,7 +25,8 @@ Options: ``q_rank`` (the queries go through a latent of their own: c_q = rmsnorm
 a ``position`` part (a head's query is [dim plain | rot_dim rotated]; W_dkv has ``rot_dim`` more rows, which are not normed
 and are one rotated key part for all heads; score = (q_plain . W_uk c + q_rot . k_rot) * scale; the cached row is
 [k_rot rotated | c], the rotated part first so that the rotation's kernel finds it at a head's start, and the matrices
-that fold and expand carry an identity block that passes it through); ``gate_activation`` None (no output gate).
+that fold and expand carry an identity block that passes it through); ``gate_activation`` None (no output gate);
+``window`` n (position i sees j only if 0 <= i - j < n; the cache keeps the window only).
 
 ``shares_latent``: the mixer has no W_dkv; its schedule entry reads the cache of an earlier entry (another layer's
 latents, written earlier in the same step) with its own W_uk, W_uv, queries, gate and output product.
@@ -46,7 +47,10 @@ class LatentAttention(Part):
 
     def __init__(self, hidden_size: int, num_heads: int, head_dim: int, value_dim: int, kv_rank: int, scale: float,
                  eps: float, shares_latent: bool = False, gate_activation: str | None = "sigmoid", q_rank: int | None = None,
-                 rot_dim: int = 0, position=None):
+                 rot_dim: int = 0, position=None, window: int | None = None):
+        if window is not None and window < 1:
+            raise ValueError(f"window must be positive, got {window}")
+        self.window = window
         if min(num_heads, head_dim, value_dim, kv_rank) < 1:
             raise ValueError("heads, widths and the latent's size must be positive")
         if rot_dim < 0 or rot_dim % 2 or (rot_dim > 0) != (position is not None):
@@ -92,7 +96,7 @@ class LatentAttention(Part):
         return specs
 
     def cache_need(self) -> CacheNeed:
-        return CacheNeed(1, self.width)
+        return CacheNeed(1, self.width, self.window)
 
     def state_need(self):
         return None
@@ -200,7 +204,7 @@ class LatentAttention(Part):
                                        *angles, None, None, kv.layer_offset, kv.page_size, kv.page_stride, H, 0, Rp, ctx.act,
                                        runs=b.runs(), amplitude=amp)
         mixed = ops.attention(folded, kv.k_pages, kv.v_pages, kv.layer_offset, b.positions, b.slot_of_token, kv.table,
-                              kv.page_size, kv.page_stride, H, 1, Rp, None, self.scale, ctx.act, runs=b.runs())
+                              kv.page_size, kv.page_stride, H, 1, Rp, self.window, self.scale, ctx.act, runs=b.runs())
         out = ops.head_gemm(mixed, self.expand_weight, ctx.act, out_act=True, gate=gate,
                             **({} if gate is None else {"activation": self.gate_activation}))
         return ops.gemm(out, self.out_weight, ctx.act, partial_sums=True)
@@ -238,7 +242,7 @@ class LatentAttention(Part):
             queries = ops.rope_kv_write(q, b.positions, b.slot_of_token, table, *angles, None, None, 0, kv.page_size, stride,
                                         H, 0, D, ctx.act, runs=runs, amplitude=amp)
         mixed = ops.attention(queries, pages[0], pages[1], 0, b.positions, b.slot_of_token, table,
-                              kv.page_size, stride, H, H, D, None, self.scale, ctx.act, runs=runs,
+                              kv.page_size, stride, H, H, D, self.window, self.scale, ctx.act, runs=runs,
                               value_width=-(-self.value_dim // 16) * 16)
         if gate is not None:
             ops.gate_rows(mixed, gate, self.gate_activation, ctx.act)

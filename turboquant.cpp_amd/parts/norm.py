@@ -2,6 +2,10 @@
 
 ``out = (v * (1 / sqrt(mean(v^2) + eps))) * weight`` with ``v = x + pending``, everything in float32
 (/root/reference/src/engine/tq_ops.c:1373-1410; a plain weight, no ``+1``).
+
+``offset`` c and ``mult`` m, for designs that store their norm weights around zero or scale what a norm lets into the
+stream: the norm multiplies by ``m (c + weight)``.  The product is formed once, in float32, when the weights are placed,
+so every kernel that takes a norm's weights takes these as they are.
 """
 from __future__ import annotations
 
@@ -12,9 +16,15 @@ from .base import ParamSpec, Part, register_part
 @register_part("norm", "rmsnorm")
 class RMSNorm(Part):
     graph_safe = True
-    def __init__(self, size: int, eps: float):
-        self.size, self.eps = size, eps
+    def __init__(self, size: int, eps: float, offset: float = 0.0, mult: float = 1.0):
+        self.size, self.eps, self.offset, self.mult = size, eps, float(offset), float(mult)
         self.weight = None
+        self._folded = False
+
+    def prepare(self, device, act):
+        if not self._folded and (self.offset != 0.0 or self.mult != 1.0):
+            self.weight = ((self.weight.float() + self.offset) * self.mult).contiguous()
+        self._folded = True
 
     def param_specs(self):
         return {"weight": ParamSpec((self.size,), role="scale")}

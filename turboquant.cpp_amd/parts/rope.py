@@ -28,7 +28,9 @@ class RotaryEncoding(Part):
     graph_safe = True
     amplitude = 1.0          # a factor on every sine and cosine (other encodings scale them)
 
-    def __init__(self, head_dim: int, rotary_dim: int, theta: float, pairing: str = "half"):
+    def __init__(self, head_dim: int, rotary_dim: int, theta: float, pairing: str = "half", double_table: bool = False):
+        """``double_table``: the frequencies are worked out in double precision and rounded once, instead of in float32."""
+        self.double_table = double_table
         if pairing not in PAIRINGS:
             raise ValueError(f"unknown pairing {pairing!r}; known: {sorted(PAIRINGS)}")
         if rotary_dim % 2 or not 0 <= rotary_dim <= head_dim:
@@ -41,6 +43,9 @@ class RotaryEncoding(Part):
         return PAIRINGS[self.pairing]
 
     def frequencies(self) -> np.ndarray:
+        if self.double_table:
+            i = np.arange(self.rotary_dim // 2, dtype=np.float64)
+            return np.power(float(self.theta), -2.0 * i / max(self.rotary_dim, 1)).astype(np.float32)
         i = np.arange(self.rotary_dim // 2, dtype=np.float32)
         expo = (np.float32(2.0) * i) / np.float32(self.rotary_dim)
         return (np.float32(1.0) / np.power(np.float32(self.theta), expo, dtype=np.float32)).astype(np.float32)
@@ -73,6 +78,31 @@ class NoRotation(Part):
 
     def prepare(self, device, act):
         self.table(device)
+
+
+@register_part("position", "llama3_rope")
+class Llama3RotaryEncoding(RotaryEncoding):
+    """Rotary encoding whose slow pairs are slowed down further, by wavelength, for sequences longer than the ``original``
+    length.  With f_i = theta^(-2i / rotary_dim) and the pair's wavelength l = 2 pi / f_i: f_i stays where
+    l < original / high; it becomes f_i / factor where l > original / low; in between, with
+    s = (original / l - low) / (high - low), it becomes (1 - s) f_i / factor + s f_i.  The table is worked out in double
+    precision and rounded once; nothing else of the rotation changes."""
+
+    def __init__(self, head_dim: int, rotary_dim: int, theta: float, factor: float, original: float, low: float, high: float,
+                 pairing: str = "half"):
+        super().__init__(head_dim, rotary_dim, theta, pairing)
+        if not (factor > 0 and original > 0 and low > 0 and high > low and theta > 0):
+            raise ValueError("the stretched rotation needs positive factor, theta, original and low, and high above low")
+        self.factor, self.original, self.low, self.high = float(factor), float(original), float(low), float(high)
+
+    def frequencies(self) -> np.ndarray:
+        i = np.arange(self.rotary_dim // 2, dtype=np.float64)
+        f = np.power(float(self.theta), -2.0 * i / max(self.rotary_dim, 1))
+        length = 2.0 * math.pi / f
+        s = (self.original / length - self.low) / (self.high - self.low)
+        out = np.where(length < self.original / self.high, f,
+                       np.where(length > self.original / self.low, f / self.factor, (1.0 - s) * f / self.factor + s * f))
+        return out.astype(np.float32)
 
 
 @register_part("position", "yarn_rope")
