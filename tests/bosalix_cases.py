@@ -133,8 +133,44 @@ def random_weights(cfg: dict, seed: int, dtype=torch.float32) -> dict[str, torch
             a = 2.0 * rng.standard_normal(shape) / np.sqrt(shape[-1])
         else:
             a = rng.standard_normal(shape) / np.sqrt(shape[-1])
-        out[name] = torch.from_numpy(np.asarray(a)).to(dtype)
+        out[name] = torch.from_numpy(np.asarray(a, dtype=np.float64)).to(torch.bfloat16).to(dtype)      # bfloat16 numbers, whatever the type
     return out
+
+
+def tokens(cfg: dict, n: int, seed: int) -> list[int]:
+    """Token ids from 2 on (0 and 1 are kept for the tests that plant a token)."""
+    rng = np.random.default_rng(1000 + seed)
+    return [int(t) for t in rng.integers(2, cfg["vocab"], size=n)]
+
+
+def random_case(seed: int) -> dict:
+    """A configuration drawn at random: two to four layers of either kind with sizes of many kinds."""
+    rng = np.random.default_rng(seed)
+    pick = lambda *xs: xs[int(rng.integers(len(xs)))]
+    width = pick(24, 40, 64, 72, 128)
+    layers, mixing = [], None
+    for _ in range(int(rng.integers(2, 5))):
+        f = pick(None, moe(pick(1, 3, 4, 8), 1, pick(8, 20, 32), identity=pick(None, 0, 1, 3)))
+        if f is not None:
+            f["router"]["top"] = int(rng.integers(1, f["router"]["experts"] + f["router"].get("identity", 0) + 1))
+        if rng.random() < 0.5:
+            rot = pick(2, 4, 8, 16)
+            layers.append((latent(pick(1, 2, 3, 4), pick(4, 8, 16, 24), rot, pick(4, 8, 16, 20), pick(6, 16, 24, 40), pick(5, 8, 16, 24),
+                                  scale=pick(0.1, 0.25, 1.0), base=pick(100.0, 10000.0), window=pick(None, 1, 7, 64, 65, 100)), f))
+        else:
+            kv = pick(1, 2)
+            dim = pick(4, 8, 16, 32, 48)
+            mix = bool(rng.random() < 0.6)
+            vdim = pick(4, 8, 16, 24) if not mix or mixing is None else mixing[1]
+            kv = kv if not mix or mixing is None else mixing[0]
+            if mix and mixing is None:
+                mixing = (kv, vdim)
+            window = pick(None, 2, 9, 64, 65, 90)
+            layers.append((attention(kv * pick(1, 2, 3), kv, dim, vdim, scale=pick(0.1, 0.3, 1.0), rot=pick(0, 2, dim // 2, dim),
+                                     base=pick(50.0, 10000.0), scaling=pick(None, stretch(pick(2.0, 8.0), pick(16, 64), 1.0, pick(2.0, 4.0))),
+                                     window=window, keep_first=pick(None, 0, 1, 4, 70), v_mix=mix), f))
+    return config(width, int(rng.integers(30, 200)), layers, eps=pick(1e-6, 1e-5), embedding_scale=pick(1.0, 4.0, 0.5),
+                  residual_mult=pick(1.0, 0.5, 0.3))
 
 
 def write_model_dir(path: str, cfg: dict, weights: dict[str, torch.Tensor]) -> str:
