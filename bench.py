@@ -28,6 +28,13 @@ does it for the Beronex design (norms around every part; attention over a latent
 the queries; lightning attention; windowed attention with head norms behind a YaRN rotation, a gate per head and layers on
 another layer's keys and values; dense gated feed-forwards and clamped experts in turn) beside Qwen2-MoE with dense
 feed-forwards and experts in turn.
+
+    python bench.py --design bosalix [--design-sizes small,medium] [--layers 8]
+
+does it for the Bosalix design (a norm on every part's output only and a mixer input blended with the token before;
+windowed attention over a latent with a rotated key part; attention with head norms, unit values mixed between layers,
+sigmoid weights and a window that keeps the first positions in sight; experts of two matrices chosen by corrected scores,
+some of them the identity) beside Qwen2-MoE with experts in every layer and as many weights.
 """
 from __future__ import annotations
 
@@ -337,6 +344,27 @@ def beronex_config(z: dict, layers: int, max_positions: int) -> dict:
             "embedding": {"scale": 1.0}, "layers": out}
 
 
+def bosalix_config(z: dict, layers: int, max_positions: int) -> dict:
+    """`layers` layers in the order latent attention, latent attention, attention, attention (the attention layers mix their
+    values with the first one's), all with a window of 1,024, every one followed by routed experts of two matrices (half as
+    wide again as the gated experts beside them, so that a layer has as many weights) with a quarter as many identity experts.
+    The cached row of a latent layer is the latent and the rotated part, 512 numbers at most."""
+    H, G, D = z["heads"], z["kv_heads"], z["dim"]
+    moe = {"kind": "moe", "router": {"experts": z["experts"], "identity": z["experts"] // 4, "top": z["top"]},
+           "expert": {"ff": z["ff"] * 3 // 2}}
+    rank = min(z["kv_rank"], 512 - D // 2)
+    kinds = [
+        ("latent_attention", {"heads": H, "dim": D, "rot_dim": D // 2, "vdim": D, "kv_rank": rank, "q_rank": 3 * z["kv_rank"] // 2,
+                              "scale": (D + D // 2) ** -0.5, "mask": {"size": 1024}, "rot": {"dims": D // 2, "base": 1e4}}),
+        ("attention", {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "mask": {"size": 1024, "keep_first": 4},
+                       "v_mix": True, "rot": {"dims": D // 2, "base": 1e6,
+                                              "scaling": {"factor": 8.0, "original": 4096, "low": 1.0, "high": 4.0}}}),
+    ]
+    out = [{"type": kinds[i % 4 // 2][0], "mixer": dict(kinds[i % 4 // 2][1]), "mlp": moe} for i in range(layers)]
+    return {"architecture": "Bosalix", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-5}, "residual_mult": 0.5,
+            "embedding": {"scale": 1.0}, "layers": out}
+
+
 def qwen_mixed_config_like(z: dict, layers: int, max_positions: int) -> dict:
     """Qwen2-MoE's layers with the dense gated feed-forward in every other layer and routed experts in the rest."""
     return dict(qwen_config_like(z, layers, max_positions), intermediate_size=z["dense_ff"],
@@ -361,7 +389,8 @@ def design_comparison(args) -> int:
     context, prompts_at, batches = 2048, (512, 2048), (1, 8)
     design = {"felepel": ("Felepel", felepel_config, qwen_config_like),
               "taminex": ("Taminex", taminex_config, qwen_dense_config_like),
-              "beronex": ("Beronex", beronex_config, qwen_mixed_config_like)}[args.design]
+              "beronex": ("Beronex", beronex_config, qwen_mixed_config_like),
+              "bosalix": ("Bosalix", bosalix_config, qwen_config_like)}[args.design]
     out = {"metric": f"{design[0]} beside Qwen2-MoE at equal sizes: prompt and decode tok/s, and milliseconds by kernel",
            "unit": "tok/s", "dtype": short, "layer_runs": layers, "data": "synthetic", "sizes": {}}
 
@@ -465,7 +494,7 @@ def main() -> int:
     ap.add_argument("--seed", type=int, default=None)
     ap.add_argument("--no-workloads", action="store_true",
                     help="leave out the two workloads of unequal prompts that the default run adds under \"workloads\"")
-    ap.add_argument("--design", default=None, choices=["felepel", "taminex", "beronex"],
+    ap.add_argument("--design", default=None, choices=["felepel", "taminex", "beronex", "bosalix"],
                     help="time this design beside Qwen2-MoE at equal sizes instead of the default workload")
     ap.add_argument("--design-sizes", default="small,medium", help="of " + ", ".join(DESIGN_SIZES))
     args = ap.parse_args()

@@ -63,7 +63,10 @@ def check(got, want, dtype="float32", what=""):
         assert e.max() < 0.25 and np.quantile(e, 0.9) < 0.08 and np.median(e) < 0.04, \
             f"{what}: median {np.median(e):.3f}, 90 % {np.quantile(e, 0.9):.3f}, worst {e.max():.3f} at {int(e.argmax())}"
     else:       # "same path": the engine against itself on another schedule, in bfloat16
-        assert np.quantile(e, 0.9) < 0.03 and e.max() < 0.3, \
+        # (a position in a hundred may stand out: where two choice scores of a router lie closer than the rounding of what
+        # feeds them, another schedule's products may choose the other expert; the float32 runs of the same tests hold every
+        # position to 1e-4)
+        assert np.quantile(e, 0.9) < 0.03 and (e > 0.3).sum() <= max(1, len(e) // 100) and e.max() < 0.6, \
             f"{what}: 90 % {np.quantile(e, 0.9):.3f}, position {int(e.argmax())} differs by {e.max():.2e}"
 
 
@@ -517,7 +520,8 @@ def test_sigmoid_weights_and_kept_positions_in_every_attention_kernel():
     nh, nkv, hd, page = 4, 2, 32, 64
     for dtype, tol in (("float32", 2e-5), ("bfloat16", 0.03)):
         adt = torch.float32 if dtype == "float32" else torch.bfloat16
-        for window, keep, n_old, n_new in ((40, 6, 300, 70), (64, 70, 200, 1), (None, 0, 100, 30), (130, 1, 500, 1), (5, 128, 190, 66)):
+        for window, keep, n_old, n_new in ((40, 6, 300, 70), (64, 70, 200, 1), (None, 0, 100, 30), (130, 1, 500, 1), (5, 128, 190, 66),
+                                           (130, 70, 4300, 1), (200, 5, 4200, 40), (70, 200, 4100, 1)):
             n = n_old + n_new
             k = rng.standard_normal((n, nkv, hd))
             v = rng.standard_normal((n, nkv, hd))
@@ -570,6 +574,35 @@ def test_greedy_generation_through_the_entry_point(made):
         for j, tok in enumerate(g):          # every chosen token is the plain model's best (or within rounding of it)
             row = rows[len(p) - 1 + j]
             assert row[tok] >= row.max() - 1e-4 * np.abs(row).max(), (p[:3], j)
+
+
+def test_a_conversation_over_state_and_kept_positions(made, tmp_path):
+    """``Model.chat``: a turn that goes on runs only the new tokens; a history that parts from the cached tokens starts over
+    (the row that a layer keeps of the token before has no earlier value); a saved conversation, with the pages of its
+    windows and of its kept first positions and its rows of state, goes on in another model object with the same tokens."""
+    from turboquant_cpp_amd import Model
+    d, cfg, w = made("wide")
+    opts = dict(dtype="float32", temperature=0.0, rep_penalty=1.0, max_tokens=5, context_length=512)
+    h1, extra, other, more = (tokens(cfg, n, 70 + n) for n in (150, 9, 150, 5))
+    with Model(d, **opts) as m, Model(d, **opts) as fresh:
+        brought = []
+        step = m.engine.step
+        m.engine.step = lambda slots, toks, *a, **k: (brought.append(len(toks[0])), step(slots, toks, *a, **k))[1]
+        out1 = m.chat(h1)
+        assert out1 == fresh.generate([h1])[0] and brought[0] == 150
+        del brought[:]
+        h2 = h1 + out1 + extra
+        out2 = m.chat(h2)
+        assert brought[0] == 1 + len(extra) and out2 == fresh.generate([h2])[0]
+        saved = str(tmp_path / "talk.kv")
+        m.save_context(saved)
+        del brought[:]
+        h3 = h1[:40] + other
+        assert m.chat(h3) == fresh.generate([h3])[0] and brought[0] == len(h3)
+        with Model(d, **opts) as later:
+            later.load_context(saved)
+            h4 = h2 + out2 + more
+            assert later.chat(h4) == fresh.generate([h4])[0]
 
 
 def test_command_line(made):

@@ -72,6 +72,9 @@ struct ColMod {
   bool biased;
   float scale, cap;
   float r1[QG], r2[QG];
+  bool sig;             // weights are sigmoids of score + pb, not normalised
+  float pb[QG];
+  int keep;             // first positions that stay visible whatever the window
 };
 template <int QG, bool MOD>
 __device__ __forceinline__ ColMod<QG, MOD> col_mod(const AttnArgs& a, const int (&head)[QG]) {
@@ -84,6 +87,10 @@ __device__ __forceinline__ ColMod<QG, MOD> col_mod(const AttnArgs& a, const int 
     m.r1[g] = m.biased ? a.mod.r1[head[g]] : 0.f;
     m.r2[g] = m.biased ? a.mod.r2[head[g]] : 0.f;
   }
+  m.sig = MOD && a.mod.pb != nullptr;
+  m.keep = MOD ? a.mod.keep : 0;
+#pragma unroll
+  for (int g = 0; g < QG; ++g) m.pb[g] = m.sig ? a.mod.pb[head[g]] : 0.f;
   return m;
 }
 
@@ -175,7 +182,7 @@ __device__ __forceinline__ void softmax_tile(f32x4 (&s)[QG][4], f32x4 (&o)[QG][D
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
           const int key = pos0 + 32 * (jt / 2) + 8 * c + 4 * (jt % 2) + v;
-          const bool ok = key <= p_q[g] && key >= lo_q[g];
+          const bool ok = MOD ? sees(key, p_q[g], lo_q[g], cm.keep) : (key <= p_q[g] && key >= lo_q[g]);
           s[g][jt][v] = ok ? s[g][jt][v] : -INFINITY;
           m_tile = fmaxf(m_tile, s[g][jt][v]);
         }
@@ -184,6 +191,23 @@ __device__ __forceinline__ void softmax_tile(f32x4 (&s)[QG][4], f32x4 (&o)[QG][D
       for (int jt = 0; jt < 4; ++jt)
 #pragma unroll
         for (int v = 0; v < 4; ++v) m_tile = fmaxf(m_tile, s[g][jt][v]);
+    }
+    if constexpr (MOD) {
+      if (cm.sig) {
+        // sigmoid weights: 1 / (1 + e^-(s + pb)); a masked score of -inf gives 1 / inf = 0.  The running maximum stays at
+        // 0, where it started, so nothing that came before is rescaled, and the sum is kept but never divided by.
+        float l_sig = 0.f;
+#pragma unroll
+        for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const float p = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-LOG2E * (s[g][jt][v] + cm.pb[g])));
+            s[g][jt][v] = p;
+            l_sig += p;
+          }
+        l_run[g] += group_sum(l_sig);
+        continue;
+      }
     }
     m_tile = group_max(m_tile) * scale2;
     const float m_new = fmaxf(m_run[g], m_tile);
@@ -488,10 +512,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DT > 16 ? 1
       m_run[g] = a.mod.sink[h] * LOG2E;
       l_run[g] = 1.f;
     }
+    if (MOD && a.mod.pb) m_run[g] = 0.f;
   }
   // tiles the workgroup goes through, and those among them that this wave's tokens can see
   const int wg_first = start + qb, wg_last = start + min(qb + 4 * QW, n) - 1;
-  const int tile_beg = reach_lo(wg_first, a.window, a.mod.chunk) / TILE, tile_end = wg_last / TILE + 1;
+  // (kept first positions: their tiles come first, then the walk jumps to the first tile of the workgroup's windows)
+  const int kept = MOD ? keep_tiles(a.mod.keep, TILE) : 0;
+  const int lo_tile = reach_lo(wg_first, a.window, a.mod.chunk) / TILE;
+  const int tile_beg = first_tile(lo_tile, kept), tile_end = wg_last / TILE + 1;
+  auto after = [&](int t) { return next_tile(t, lo_tile, kept); };
   const int wq0 = qb + wave * QW;
   const bool wave_has = wq0 < n;
   const int wave_first = start + wq0, wave_last = start + min(wq0 + QW, n) - 1;
@@ -531,7 +560,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DT > 16 ? 1
   u32x4 pk[KCH], pv[VCH];
   const int tiles_per_page = a.page_size / TILE;
   int page_next = table[tile_beg / tiles_per_page];     // page of the tile that the next fetch takes
-#define TQ_FETCH(tile)                                                                                      \
+#define TQ_FETCH(tile, nxt)                                                                                 \
   do {                                                                                                      \
     const int64_t base = head_off + (int64_t)page_next * a.page_stride;                                     \
     const int in_page = ((tile) % tiles_per_page) * TILE;                                                   \
@@ -539,7 +568,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DT > 16 ? 1
     const bf16_t* vg = a.v_pool + base + in_page;                                                           \
     _Pragma("unroll") for (int j = 0; j < KCH; ++j) pk[j] = *reinterpret_cast<const u32x4*>(kg + k_g(j));   \
     _Pragma("unroll") for (int j = 0; j < VCH; ++j) pv[j] = *reinterpret_cast<const u32x4*>(vg + v_g(j));   \
-    if ((tile) + 1 < tile_end) page_next = table[((tile) + 1) / tiles_per_page];                            \
+    if ((nxt) < tile_end) page_next = table[(nxt) / tiles_per_page];                                        \
   } while (0)
 #define TQ_STAGE(off)                                                                                       \
   do {                                                                                                      \
@@ -547,13 +576,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DT > 16 ? 1
     _Pragma("unroll") for (int j = 0; j < VCH; ++j) *reinterpret_cast<u32x4*>(Vs + (off) + v_l(j)) = pv[j]; \
   } while (0)
 
-  TQ_FETCH(tile_beg);
+  TQ_FETCH(tile_beg, after(tile_beg));
   if constexpr (ONEBUF) {
-    for (int tile = tile_beg; tile < tile_end; ++tile) {
+    for (int tile = tile_beg; tile < tile_end; tile = after(tile)) {
+      const int t1 = after(tile);
       TQ_STAGE(0);
-      if (tile + 1 < tile_end) TQ_FETCH(tile + 1);
+      if (t1 < tile_end) TQ_FETCH(t1, after(t1));
       __syncthreads();
-      if (tile >= wave_beg && tile < wave_end) {
+      if ((tile >= wave_beg || tile < kept) && tile < wave_end) {
         const int pos0 = tile * TILE;
         const bool masked = pos0 + TILE - 1 > wave_first || pos0 < wave_lo_last;
         tile_step<DT, QG, EXACT, EXACT, false, MOD, VD>(o, m_run, l_run, qf, Ks, kstr, Vs, vstr, hd, pos0, p_q, lo_q,
@@ -563,15 +593,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DT > 16 ? 1
     }
   } else {
   TQ_STAGE(0);
-  if (tile_beg + 1 < tile_end) TQ_FETCH(tile_beg + 1);
+  if (after(tile_beg) < tile_end) TQ_FETCH(after(tile_beg), after(after(tile_beg)));
   __syncthreads();
   int cur = 0;
-  for (int tile = tile_beg; tile < tile_end; ++tile, cur ^= buf) {
-    if (tile + 1 < tile_end) {
+  for (int tile = tile_beg; tile < tile_end; tile = after(tile), cur ^= buf) {
+    const int t1 = after(tile), t2 = after(t1);
+    if (t1 < tile_end) {
       TQ_STAGE(cur ^ buf);
-      if (tile + 2 < tile_end) TQ_FETCH(tile + 2);
+      if (t2 < tile_end) TQ_FETCH(t2, after(t2));
     }
-    if (tile >= wave_beg && tile < wave_end) {
+    if ((tile >= wave_beg || tile < kept) && tile < wave_end) {
       const int pos0 = tile * TILE;
       const bool masked = pos0 + TILE - 1 > wave_first || pos0 < wave_lo_last;
       tile_step<DT, QG, EXACT, EXACT, false, MOD, VD>(o, m_run, l_run, qf, Ks + cur, kstr, Vs + cur, vstr, hd, pos0, p_q, lo_q,
@@ -585,7 +616,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DT > 16 ? 1
 #pragma unroll
   for (int g = 0; g < QG; ++g) {
     if (p_q[g] < 0) continue;
-    float inv = 1.0f / l_run[g];
+    float inv = (MOD && a.mod.pb) ? 1.0f : 1.0f / l_run[g];
     if (a.head_gate) inv /= 1.0f + expf(-a.head_gate[(size_t)(t0 + p_q[g] - start) * a.ld_gate + h]);
     bf16_t* orow = a.out + ((size_t)(t0 + p_q[g] - start) * a.nh + h) * hd;
 #pragma unroll
@@ -637,19 +668,28 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(AHEAD ? 1 : 
 
   bf16x8 qf[1][(DT + 1) / 2];
   load_query<DT>(qf[0], a.q + ((size_t)t * a.nh + h) * a.hd, a.hd, valid);
+  // tiles of kept first positions that lie before the window's first tile: a run takes its share of them before its
+  // share of the window's tiles
+  const int kept_before = MOD ? min(keep_tiles(a.mod.keep, TILE), lo / TILE) : 0;
   for (int run = blockIdx.x; run < n_runs; run += gridDim.x) {
     const int tile_beg = max(run * S, lo / TILE), tile_end = min((run + 1) * S, p / TILE + 1);
-    if (tile_beg >= tile_end) continue;       // all of the run lies before the window
+    const int kept_beg = run * S, kept_end = min(tile_end, kept_before);
+    if (tile_beg >= tile_end && kept_beg >= kept_end) continue;       // all of the run lies before the window
     f32x4 o[1][VD];
 #pragma unroll
     for (int dt = 0; dt < VD; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float m_run[1] = {-INFINITY}, l_run[1] = {0.f};
-    if constexpr (AHEAD)
-      attend_ahead<DT, MOD>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride,
-                       tile_beg, tile_end, p, valid, lo, a.scale * LOG2E, cm);
-    else
-      attend<DT, EXACT, MOD, VD>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride,
-                        a.hd, tile_beg, tile_end, p, valid, lo, a.scale * LOG2E, cm, dt0);
+    float m_run[1] = {(MOD && a.mod.pb) ? 0.f : -INFINITY}, l_run[1] = {0.f};
+#pragma unroll
+    for (int part = MOD ? 0 : 1; part < 2; ++part) {
+      const int beg = part ? tile_beg : kept_beg, end = part ? tile_end : kept_end;
+      if (beg >= end) continue;
+      if constexpr (AHEAD)
+        attend_ahead<DT, MOD>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride,
+                         beg, end, p, valid, lo, a.scale * LOG2E, cm);
+      else
+        attend<DT, EXACT, MOD, VD>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride,
+                          a.hd, beg, end, p, valid, lo, a.scale * LOG2E, cm, dt0);
+    }
     if (!valid) continue;
     float* out = a.partial + (((size_t)b * a.nh + h) * a.max_runs + run) * (a.hd + 2);
 #pragma unroll
@@ -679,39 +719,47 @@ __global__ __launch_bounds__(256) void attn_join_kernel(AttnArgs a) {
   const int p = a.start[b];
   const int lo = reach_lo(p, a.window, a.mod.chunk);
   const int S = tiles_per_run(p);
-  const int run_beg = lo / TILE / S, run_end = p / TILE / S + 1;
+  int run_beg = lo / TILE / S;
+  const int run_end = p / TILE / S + 1;
+  // runs that hold kept first positions before the window's first tile come first, then the window's runs: entry i of
+  // the walk is run RUN_OF(i)
+  int kept_runs = (min(keep_tiles(a.mod.keep, TILE), lo / TILE) + S - 1) / S;
+  if (kept_runs >= run_beg) run_beg = kept_runs = 0;
+  const int n_runs = kept_runs + run_end - run_beg;
+#define RUN_OF(i) ((i) < kept_runs ? (i) : run_beg + (i) - kept_runs)
   const int stride = a.hd + 2;
   const float* part = a.partial + ((size_t)b * a.nh + h) * a.max_runs * stride;
   float m = -INFINITY;
-  for (int s = run_beg + lane; s < run_end; s += 64) m = fmaxf(m, part[(size_t)s * stride + a.hd]);
+  for (int i = lane; i < n_runs; i += 64) m = fmaxf(m, part[(size_t)RUN_OF(i) * stride + a.hd]);
   m = wave_max(m);
   float l = 0.f;
   if (a.mod.sink) {         // the sink joins here, once, like one more run with a sum of 1 and no values
     m = fmaxf(m, a.mod.sink[h] * LOG2E);
     l = __builtin_amdgcn_exp2f(a.mod.sink[h] * LOG2E - m);
   }
-  for (int s0 = run_beg; s0 < run_end; s0 += 64) {     // denominators in run order, 64 runs at a time
-    const int s = s0 + lane;
+  for (int i0 = 0; i0 < n_runs; i0 += 64) {     // denominators in run order, 64 runs at a time
+    const int i = i0 + lane;
     float w = 0.f, wl = 0.f;
-    if (s < run_end) {
-      w = __builtin_amdgcn_exp2f(part[(size_t)s * stride + a.hd] - m);      // maxima are in units of log2
-      wl = w * part[(size_t)s * stride + a.hd + 1];
-      wgt[s - run_beg] = w;
+    if (i < n_runs) {
+      const size_t s = RUN_OF(i);
+      w = __builtin_amdgcn_exp2f(part[s * stride + a.hd] - m);      // maxima are in units of log2
+      wl = w * part[s * stride + a.hd + 1];
+      wgt[i] = w;
     }
     l += wave_sum(wl);
   }
   __builtin_amdgcn_wave_barrier();
-  float inv = 1.0f / l;
+  float inv = a.mod.pb ? 1.0f : 1.0f / l;       // sigmoid weights are not normalised (every run's maximum is 0)
   if (a.head_gate) inv /= 1.0f + expf(-a.head_gate[(size_t)a.cu_seqlens[b] * a.ld_gate + h]);
   bf16_t* orow = a.out + ((size_t)a.cu_seqlens[b] * a.nh + h) * a.hd;
   if (a.hd % 128 == 0) {      // a lane takes two neighbouring dimensions of its wave's 128: one pass over the runs, 8 bytes at a time
     const int d = 128 * wave + 2 * lane;
     float acc0 = 0.f, acc1 = 0.f;
 #pragma unroll 8
-    for (int s = run_beg; s < run_end; ++s) {
-      const float2 v = *reinterpret_cast<const float2*>(part + (size_t)s * stride + d);
-      acc0 = fmaf(wgt[s - run_beg], v.x, acc0);
-      acc1 = fmaf(wgt[s - run_beg], v.y, acc1);
+    for (int i = 0; i < n_runs; ++i) {
+      const float2 v = *reinterpret_cast<const float2*>(part + (size_t)RUN_OF(i) * stride + d);
+      acc0 = fmaf(wgt[i], v.x, acc0);
+      acc1 = fmaf(wgt[i], v.y, acc1);
     }
     *reinterpret_cast<uint32_t*>(orow + d) = pack2(acc0 * inv, acc1 * inv);
     return;
@@ -719,9 +767,10 @@ __global__ __launch_bounds__(256) void attn_join_kernel(AttnArgs a) {
   for (int d = lane; d < a.hd; d += 64) {
     float acc = 0.f;
 #pragma unroll 8
-    for (int s = run_beg; s < run_end; ++s) acc = fmaf(wgt[s - run_beg], part[(size_t)s * stride + d], acc);
+    for (int i = 0; i < n_runs; ++i) acc = fmaf(wgt[i], part[(size_t)RUN_OF(i) * stride + d], acc);
     orow[d] = f32_to_bf16(acc * inv);
   }
+#undef RUN_OF
 }
 
 // ------------------------------------------------------------------------------------------ launch
@@ -738,7 +787,7 @@ static int launch_prefill_as(const AttnArgs& a, int B, int max_new, hipStream_t 
 // (the kernels that cap or bias scores are instantiations of their own, so that the others carry nothing of it)
 template <int DT, int QG, bool EXACT, int VD = DT>
 static int launch_prefill(const AttnArgs& a, int B, int max_new, hipStream_t st) {
-  return (a.mod.cap > 0.f || a.mod.r1) ? launch_prefill_as<DT, QG, EXACT, true, VD>(a, B, max_new, st)
+  return (a.mod.cap > 0.f || a.mod.r1 || a.mod.pb || a.mod.keep > 0) ? launch_prefill_as<DT, QG, EXACT, true, VD>(a, B, max_new, st)
                                        : launch_prefill_as<DT, QG, EXACT, false, VD>(a, B, max_new, st);
 }
 template <int DT, bool EXACT, bool MOD>
@@ -760,7 +809,7 @@ static void launch_decode_as(const AttnArgs& a, int B, int grid_runs, hipStream_
 }
 template <int DT, bool EXACT>
 static void launch_decode(const AttnArgs& a, int B, int grid_runs, hipStream_t st) {
-  if (a.mod.cap > 0.f || a.mod.r1) launch_decode_as<DT, EXACT, true>(a, B, grid_runs, st);
+  if (a.mod.cap > 0.f || a.mod.r1 || a.mod.pb || a.mod.keep > 0) launch_decode_as<DT, EXACT, true>(a, B, grid_runs, st);
   else launch_decode_as<DT, EXACT, false>(a, B, grid_runs, st);
 }
 
@@ -775,14 +824,16 @@ TQ_API int64_t tq_attention_decode_scratch(int B, int nh, int hd, int max_end) {
 // value_width (0: hd): the values' first numbers that matter; a head's value rows behind them are zeros, and so is the
 // output there, which lets a kernel leave them out.  head_gate (null: none), float [T][ld_gate]: the output of head h of
 // token t is multiplied by sigmoid(head_gate[t][h]) where it is normalised, before it is rounded.
-TQ_API int tq_attention_mfma_ex(const void* q, const void* k_pool, const void* v_pool, const int* block_table,
+// pb, keep: sigmoid weights with a bias per head, and first positions that stay visible (score_mod.h; null, 0: neither).
+TQ_API int tq_attention_mfma_sig(const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                                        int bt_stride, const int* cu_seqlens, const int* slots, const int* start, int page_size,
                                        int64_t page_stride, int B, int nh, int nkv, int hd, int window, float scale,
                                        float softcap, const float* r1, const float* r2, int chunk, const float* sink,
                                        void* out, float* partial, int decode, int max_new, int max_end, int value_width,
-                                       const float* head_gate, int64_t ld_gate, hipStream_t st) {
+                                       const float* head_gate, int64_t ld_gate, const float* pb, int keep, hipStream_t st) {
   if (B <= 0) return 0;
-  if ((r1 == nullptr) != (r2 == nullptr) || chunk < 0 || softcap < 0.f || value_width < 0 || value_width > hd || (head_gate && ld_gate < nh))
+  if ((r1 == nullptr) != (r2 == nullptr) || chunk < 0 || softcap < 0.f || value_width < 0 || value_width > hd || (head_gate && ld_gate < nh)
+      || keep < 0 || (pb && sink))
     return TQ_ERR_BAD_ARG;
   if (hd % 16 != 0 || hd < 16 || hd > 512 || page_size % TILE != 0 || nkv <= 0 || nh % nkv != 0)
     return TQ_ERR_UNSUPPORTED;
@@ -790,7 +841,7 @@ TQ_API int tq_attention_mfma_ex(const void* q, const void* k_pool, const void* v
   if (decode && most_runs(max_end) > MAX_RUNS_LDS) return TQ_ERR_UNSUPPORTED;
   AttnArgs a{(const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, bt_stride, cu_seqlens, slots,
              start, page_size, page_stride, nh, nkv, hd, window, scale, (bf16_t*)out, partial,
-             most_runs(max_end), ScoreMod{softcap, r1, r2, chunk, sink}, head_gate, ld_gate};
+             most_runs(max_end), ScoreMod{softcap, r1, r2, chunk, sink, pb, keep}, head_gate, ld_gate};
   const int dt = hd / 16;
   // head sizes 64, 128 and 256 have kernels of their own in which nothing depends on hd at run time
   if (decode) {
@@ -825,6 +876,17 @@ TQ_API int tq_attention_mfma_ex(const void* q, const void* k_pool, const void* v
   }
   TQ_LAUNCH_CHECK();
   return 0;
+}
+
+TQ_API int tq_attention_mfma_ex(const void* q, const void* k_pool, const void* v_pool, const int* block_table,
+                                       int bt_stride, const int* cu_seqlens, const int* slots, const int* start, int page_size,
+                                       int64_t page_stride, int B, int nh, int nkv, int hd, int window, float scale,
+                                       float softcap, const float* r1, const float* r2, int chunk, const float* sink,
+                                       void* out, float* partial, int decode, int max_new, int max_end, int value_width,
+                                       const float* head_gate, int64_t ld_gate, hipStream_t st) {
+  return tq_attention_mfma_sig(q, k_pool, v_pool, block_table, bt_stride, cu_seqlens, slots, start, page_size, page_stride, B,
+                               nh, nkv, hd, window, scale, softcap, r1, r2, chunk, sink, out, partial, decode, max_new, max_end,
+                               value_width, head_gate, ld_gate, nullptr, 0, st);
 }
 
 TQ_API int tq_attention_mfma_mod(const void* q, const void* k_pool, const void* v_pool, const int* block_table,

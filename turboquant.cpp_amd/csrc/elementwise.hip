@@ -190,7 +190,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const float* __restric
       float a = xr[i];
       if (y) {
         float acc = 0.f;
-        for (int j = 0; j < topk; ++j) acc += slot[j] < 0 ? 0.f : wgt[j] * y[(size_t)slot[j] * H + i];
+        for (int j = 0; j < topk; ++j)
+          if (slot[j] >= 0) acc += wgt[j] * y[(size_t)slot[j] * H + i];      // (-1: a pair without a row)
         if (S > 0) {
           float sh = 0.f;
           for (int s = 0; s < S; ++s) sh += dr[s * delta_stride + i];
@@ -833,7 +834,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
   const float g = gate ? gate[t] : 1.0f;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     float acc = 0.f;
-    for (int j = 0; j < topk; ++j) acc += slot[j] < 0 ? 0.f : wgt[j] * y[(size_t)slot[j] * H + i];
+    for (int j = 0; j < topk; ++j)
+      if (slot[j] >= 0) acc += wgt[j] * y[(size_t)slot[j] * H + i];      // (-1: a pair without a row)
     if (shared) {
       float sh = 0.f;
       for (int s = 0; s < S; ++s) sh += shared[s * shared_stride + (size_t)t * H + i];

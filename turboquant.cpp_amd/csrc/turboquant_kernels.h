@@ -176,6 +176,32 @@ int tq_route_biased(const float* x, const void* wr, const void* shared_w, const 
         int topk, int renorm, int groups, int keep, int* ids, float* weights, float* shared_gate, float* logits,
         int unit, int cap, int* sorted_token, int* pair_slot, int* tile_expert, int* n_tiles, int T, int H,
         hipStream_t st);
+// A router whose softmax runs over all E rows, whose choice is by score + correction and whose weights are the scores; rows
+// from n_real on are experts without matrices (the identity): pair_slot -1, id_gate[t] the sum of their weights.
+int tq_route_scored(const float* x, const void* wr, const float* correction, int wtype, int E, int n_real, int topk,
+        int* ids, float* weights, float* id_gate, float* logits, int unit, int cap, int* sorted_token, int* pair_slot,
+        int* tile_expert, int* n_tiles, int T, int H, hipStream_t st);
+// The *_sig forms of the attention entry points add what score_mod.h calls pb and keep: sigmoid weights with a bias per
+// head in the softmax's place, and first positions that stay visible whatever the window.
+int tq_attention_generic_sig(const void* q, const void* k_pool, const void* v_pool, const int* positions,
+        const int* seq_of_token, const int* block_table, int bt_stride, int page_size, int64_t page_stride, int T,
+        int nh, int nkv, int hd, int window, float scale, float softcap, const float* r1, const float* r2, int chunk,
+        const float* sink, const float* pb, int keep, void* out, hipStream_t st);
+int tq_attention_mfma_sig(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
+        const int* cu_seqlens, const int* slots, const int* start, int page_size, int64_t page_stride, int B,
+        int nh, int nkv, int hd, int window, float scale, float softcap, const float* r1, const float* r2, int chunk,
+        const float* sink, void* out, float* partial, int decode, int max_new, int max_end, int value_width,
+        const float* head_gate, int64_t ld_gate, const float* pb, int keep, hipStream_t st);
+int tq_attention_f32_sig(const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
+        const int* cu_seqlens, const int* slots, const int* start, int page_size, int64_t page_stride, int B,
+        int nh, int nkv, int hd, int window, float scale, float softcap, const float* r1, const float* r2, int chunk,
+        const float* sink, const float* pb, int keep, void* out, void* partial, int decode, int max_new, int max_end,
+        hipStream_t st);
+// elementwise.hip: a mixer input blended token by token with the row before; unit values mixed with another layer's
+int tq_token_shift(const float* x, const void* w, int wtype, float* state, const int* cu_seqlens, const int* slots,
+        int B, void* out, int T, int H, hipStream_t st);
+int tq_value_norm_mix(float* v, int64_t ld, int hd, int vd, int heads, float eps, const float* first,
+        int64_t ld_first, int hd_first, const void* lambda, int wtype, int T, hipStream_t st);
 // sampling.hip: greedy choice, negative log-likelihood, repetition penalty, temperature and top-p (both libraries; the two *_static entry points are declared in no_alloc.h)
 int tq_argmax(const float* logits, int R, int V, int* out, hipStream_t st);
 int tq_nll(const float* logits, int R, int V, const int* target, float* out, hipStream_t st);
