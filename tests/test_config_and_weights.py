@@ -122,7 +122,7 @@ def test_unknown_architecture_lists_the_known_ones():
     d["architectures"] = ["Nope"]
     with pytest.raises(ConfigError) as e:
         config_from_dict(d)
-    assert "Qwen2MoeForCausalLM" in str(e.value) and known_architectures() == ["Beronex", "Felepel", "Qwen2MoeForCausalLM", "Taminex"]
+    assert "Qwen2MoeForCausalLM" in str(e.value) and known_architectures() == ["Beronex", "Bosalix", "Felepel", "Qwen2MoeForCausalLM", "Taminex"]
 
 
 def test_config_from_dir_errors(tmp_path):
