@@ -459,6 +459,26 @@ def test_token_shift_kernel_keeps_the_last_row_per_slot():
         assert float(st[0].abs().sum() + st[2].abs().sum()) == 0.0
 
 
+def test_token_shift_behind_the_sum_of_a_decode_step():
+    """One token per sequence: the blend in the launch that sums a normed part into the stream gives the bits of the two
+    launches apart, and leaves the same rows in the slots."""
+    from turboquant_cpp_amd.csrc import ops
+    rng = np.random.default_rng(4)
+    for H in (40, 256):
+        T = 5
+        slots = torch.tensor([7, 2, 0, 5, 3], dtype=torch.int32, device="cuda")
+        runs = {"cu_seqlens": torch.arange(T + 1, dtype=torch.int32, device="cuda"), "slots": slots}
+        x, d, st = rng.standard_normal((T, H)), rng.standard_normal((2, T, H)), rng.standard_normal((8, H))
+        wn, ws = f32(1 + 0.1 * rng.standard_normal(H)), f32(rng.uniform(0, 1, H))
+        for act in ("float32", "bfloat16"):
+            xa, xb, sa, sb = f32(x), f32(x), f32(st), f32(st)
+            ha, _ = ops.add_rmsnorm(xa, ops.NormedDelta(f32(d), wn, 1e-5), None, 0.0, act, stream=True, shift=(ws, sa, slots))
+            ops.add_rmsnorm(xb, ops.NormedDelta(f32(d), wn, 1e-5), None, 0.0, act)
+            hb = ops.token_shift(xb, ws, sb, runs, act)
+            assert torch.equal(xa, xb) and torch.equal(sa, sb) and torch.equal(ha, hb)
+            assert torch.equal(sa[slots.long()], xa) and ha.data_ptr() != xa.data_ptr()
+
+
 def test_unit_values_and_their_mix():
     from turboquant_cpp_amd.csrc import ops
     rng = np.random.default_rng(1)

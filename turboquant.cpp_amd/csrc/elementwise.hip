@@ -896,7 +896,8 @@ __global__ void add_normed_rmsnorm_kernel(float* __restrict__ x, const float* __
                                           int topk, const float* __restrict__ gate, const W* __restrict__ wd,
                                           float eps_d, const W* __restrict__ w, float eps,
                                           const int* __restrict__ rows, act_t* __restrict__ out,
-                                          float* __restrict__ out32, int H) {
+                                          float* __restrict__ out32, int H, const float* __restrict__ shift_w,
+                                          float* __restrict__ shift_state, const int* __restrict__ shift_slots) {
   extern __shared__ __attribute__((aligned(16))) float v[];       // H floats, then one float per wave
   __shared__ int slot[64];
   __shared__ float wgt[64];
@@ -905,6 +906,10 @@ __global__ void add_normed_rmsnorm_kernel(float* __restrict__ x, const float* __
   const int row = rows ? rows[r] : r;
   float* xr = x + (size_t)row * H;
   const float* dr = delta + (size_t)row * H;
+  // (shift_state, with w null and every row a sequence of its own: what goes out is the summed row blended with the row
+  // that the sequence's slot keeps, a + (kept - a) * shift_w, and the slot then keeps the summed row: the token shift of a
+  // decode step, without a launch of its own)
+  float* kept = shift_state ? shift_state + (size_t)shift_slots[row] * H : nullptr;
   float g = 1.0f;
   if (y) {
     if (threadIdx.x < topk) {
@@ -972,7 +977,14 @@ __global__ void add_normed_rmsnorm_kernel(float* __restrict__ x, const float* __
       const float a = xr[i + u] + (v[i + u] * rd) * to_f32(wd[i + u]);
       v[i + u] = a;
       if (!rows) xr[i + u] = a;
-      if (!w && out) out[(size_t)r * H + i + u] = from_f32<act_t>(a);      // the summed stream itself, for a part that reads it un-normed
+      if (!w && out) {      // the summed stream itself, for a part that reads it un-normed
+        float h = a;
+        if (kept) {
+          h = a + (kept[i + u] - a) * shift_w[i + u];
+          kept[i + u] = a;
+        }
+        out[(size_t)r * H + i + u] = from_f32<act_t>(h);
+      }
       s2 += a * a;
     }
   }
@@ -989,13 +1001,31 @@ __global__ void add_normed_rmsnorm_kernel(float* __restrict__ x, const float* __
   }
 }
 
+TQ_API int tq_add_normed_rmsnorm_shift(float* x, const float* delta, int S, int64_t delta_stride, const float* y,
+                                       const int* pair_slot, const float* weights, int topk, const float* gate,
+                                       const void* wd, float eps_d, const void* w, int wtype, float eps, const int* rows,
+                                       int R, void* out, float* out32, int H, const float* shift_w, float* shift_state,
+                                       const int* shift_slots, hipStream_t st);
+
 // As tq_add_rmsnorm, with the weights wd and the eps_d of the norm that what is added passes first; w null: the
 // stream is summed and nothing is normed (no out32; `out`, if given, receives the summed stream in the activation type).
 TQ_API int tq_add_normed_rmsnorm(float* x, const float* delta, int S, int64_t delta_stride, const float* y,
                                  const int* pair_slot, const float* weights, int topk, const float* gate,
                                  const void* wd, float eps_d, const void* w, int wtype, float eps, const int* rows,
                                  int R, void* out, float* out32, int H, hipStream_t st) {
+  return tq_add_normed_rmsnorm_shift(x, delta, S, delta_stride, y, pair_slot, weights, topk, gate, wd, eps_d, w, wtype, eps, rows,
+                                     R, out, out32, H, nullptr, nullptr, nullptr, st);
+}
+
+// The same with a token shift behind the sum (w and rows null, `out` given, every row a sequence of its own whose slot is
+// shift_slots[row]): out = a + (shift_state[slot] - a) * shift_w for the summed row a, and shift_state[slot] = a.
+TQ_API int tq_add_normed_rmsnorm_shift(float* x, const float* delta, int S, int64_t delta_stride, const float* y,
+                                       const int* pair_slot, const float* weights, int topk, const float* gate,
+                                       const void* wd, float eps_d, const void* w, int wtype, float eps, const int* rows,
+                                       int R, void* out, float* out32, int H, const float* shift_w, float* shift_state,
+                                       const int* shift_slots, hipStream_t st) {
   if (R <= 0) return 0;
+  if (shift_state && (w || rows || !out || !shift_w || !shift_slots)) return TQ_ERR_BAD_ARG;
   if (!wd || (y && (topk < 1 || topk > 64 || !pair_slot || !weights))) return TQ_ERR_BAD_ARG;
   if (!y && (S < 1 || !delta)) return TQ_ERR_BAD_ARG;
   const int threads = (H % 4 == 0 && H >= 2048) ? 512 : 256;
@@ -1008,13 +1038,13 @@ TQ_API int tq_add_normed_rmsnorm(float* x, const float* delta, int S, int64_t de
         (void)hipFuncSetAttribute((const void*)add_normed_rmsnorm_kernel<W, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
       hipLaunchKernelGGL((add_normed_rmsnorm_kernel<W, true>), dim3(R), dim3(threads), shmem, st, x, delta, S,
                          (size_t)delta_stride, y, pair_slot, weights, topk, gate, (const W*)wd, eps_d, (const W*)w, eps,
-                         rows, (act_t*)out, out32, H);
+                         rows, (act_t*)out, out32, H, shift_w, shift_state, shift_slots);
     } else {
       if (shmem > 48 * 1024)
         (void)hipFuncSetAttribute((const void*)add_normed_rmsnorm_kernel<W, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
       hipLaunchKernelGGL((add_normed_rmsnorm_kernel<W, false>), dim3(R), dim3(threads), shmem, st, x, delta, S,
                          (size_t)delta_stride, y, pair_slot, weights, topk, gate, (const W*)wd, eps_d, (const W*)w, eps,
-                         rows, (act_t*)out, out32, H);
+                         rows, (act_t*)out, out32, H, shift_w, shift_state, shift_slots);
     }
   });
   TQ_LAUNCH_CHECK();
@@ -1032,8 +1062,8 @@ __global__ __launch_bounds__(256) void token_shift_kernel(const float* __restric
                                                           float* __restrict__ state, const int* __restrict__ cu_seqlens,
                                                           const int* __restrict__ slots, int B, act_t* __restrict__ out, int H) {
   const int t = blockIdx.x;
-  // the run that holds token t: the last one that starts at or before it
-  int lo = 0, hi = B - 1;
+  // the run that holds token t: the last one that starts at or before it (a step of one token per sequence: run t)
+  int lo = gridDim.x == (unsigned)B ? t : 0, hi = gridDim.x == (unsigned)B ? t : B - 1;
   while (lo < hi) {
     const int mid = (lo + hi + 1) / 2;
     if (cu_seqlens[mid] <= t) lo = mid; else hi = mid - 1;

@@ -61,6 +61,8 @@ _SIGNATURES = {
     "tq_embed_pos": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_f32, _c_ptr],
     "tq_add_normed_rmsnorm": [_c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_f32, _c_ptr,
                               _c_int, _c_f32, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
+    "tq_add_normed_rmsnorm_shift": [_c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_f32, _c_ptr,
+                                    _c_int, _c_f32, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     "tq_attention_generic_mod": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_i64, _c_int, _c_int,
                                  _c_int, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr],
     "tq_attention_generic_sig": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_i64, _c_int, _c_int,
@@ -378,13 +380,17 @@ class NormedDelta:
 
 
 def add_rmsnorm(x: torch.Tensor, delta, weight: torch.Tensor | None, eps: float, act,
-                rows: torch.Tensor | None = None, want_act: bool = True, want_f32: bool = False, stream: bool = False):
+                rows: torch.Tensor | None = None, want_act: bool = True, want_f32: bool = False, stream: bool = False,
+                shift: tuple | None = None):
     """x += delta (in place, unless ``rows`` picks rows), where delta is None, float32 partial sums [S, T, H] added
     one after the other, a GatheredSum, or a NormedDelta around either (then what is added is its RMS norm); returns
     rmsnorm(x) * weight as (activation-typed or None, float32 or None), one row per entry of ``rows`` (all rows if
     None).  ``weight`` None (with a NormedDelta only): the stream is summed and nothing is returned.  ``stream`` (with
     ``weight`` None, and delta None or a NormedDelta): the summed stream itself is returned in the activation type, for
-    a part that reads the stream un-normed (on the float32 library that is ``x``, which the next sum changes)."""
+    a part that reads the stream un-normed (on the float32 library that is ``x``, which the next sum changes).
+    ``shift`` (with ``stream`` behind a NormedDelta, in a step of one token per sequence): (weight float32 [H], state float32
+    [slots, H], slots int32 [T]); what is returned is the summed row blended with the row that the sequence's slot keeps,
+    ``a + (state[slot] - a) * weight``, and the slot then keeps the summed row: ``token_shift`` without a launch of its own."""
     k = "add_rmsnorm"
     _check(x, k, "x", torch.float32)
     _need(x.dim() == 2, k, "x must be [T, H]")
@@ -401,10 +407,20 @@ def add_rmsnorm(x: torch.Tensor, delta, weight: torch.Tensor | None, eps: float,
         _need(delta is not None, k, "a normed part needs something to norm")
     if weight is None:
         _need(post is not None and rows is None, k, "without a weight only a normed part can be summed, into all rows")
-        want_act, want_f32 = stream and dtype_name(act) != "float32", False
+        want_act, want_f32 = stream and (dtype_name(act) != "float32" or shift is not None), False
     else:
         _check(weight, k, "weight", tuple(_WTYPE), (H,))
         _need(post is None or post.weight.dtype == weight.dtype, k, "the two norms' weights must have one type")
+    shift_args = (None, None, None)
+    if shift is not None:
+        _need(stream and post is not None and post.weight.dtype == torch.float32, k,
+              "a shift rides behind the sum of a normed part whose norm weights are float32")
+        sw, sstate, sslots = shift
+        _check(sw, k, "shift weight", torch.float32, (H,))
+        _check(sstate, k, "shift state", torch.float32)
+        _need(sstate.dim() == 2 and sstate.shape[1] == H, k, lambda: f"shift state must be [slots, {H}]")
+        _check(sslots, k, "shift slots", torch.int32, (T,))
+        shift_args = (_ptr(sw), _ptr(sstate), _ptr(sslots))
     y = pair_slot = weights = gate = None
     topk = 0
     if isinstance(delta, GatheredSum):
@@ -432,10 +448,10 @@ def add_rmsnorm(x: torch.Tensor, delta, weight: torch.Tensor | None, eps: float,
     out = torch.empty((R, H), dtype=adt, device=x.device) if want_act else None
     out32 = torch.empty((R, H), dtype=torch.float32, device=x.device) if want_f32 else None
     if post is not None:
-        _run(k, library(act).tq_add_normed_rmsnorm(_ptr(x), _ptr(delta), S, stride, _ptr(y), _ptr(pair_slot), _ptr(weights),
-                                                   topk, _ptr(gate), _ptr(post.weight), float(post.eps), _ptr(weight),
-                                                   _WTYPE[post.weight.dtype], float(eps), _ptr(rows), R, _ptr(out),
-                                                   _ptr(out32), H, _stream()))
+        _run(k, library(act).tq_add_normed_rmsnorm_shift(_ptr(x), _ptr(delta), S, stride, _ptr(y), _ptr(pair_slot), _ptr(weights),
+                                                         topk, _ptr(gate), _ptr(post.weight), float(post.eps), _ptr(weight),
+                                                         _WTYPE[post.weight.dtype], float(eps), _ptr(rows), R, _ptr(out),
+                                                         _ptr(out32), H, *shift_args, _stream()))
         return (x if stream and out is None else out), out32
     _run(k, library(act).tq_add_rmsnorm(_ptr(x), _ptr(delta), S, stride, _ptr(y), _ptr(pair_slot), _ptr(weights), topk,
                                         _ptr(gate), _ptr(weight), _WTYPE[weight.dtype], float(eps), _ptr(rows), R,

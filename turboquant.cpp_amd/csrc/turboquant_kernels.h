@@ -197,6 +197,10 @@ int tq_attention_f32_sig(const void* q, const void* k_pool, const void* v_pool, 
         int nh, int nkv, int hd, int window, float scale, float softcap, const float* r1, const float* r2, int chunk,
         const float* sink, const float* pb, int keep, void* out, void* partial, int decode, int max_new, int max_end,
         hipStream_t st);
+int tq_add_normed_rmsnorm_shift(float* x, const float* delta, int S, int64_t delta_stride, const float* y, const int* pair_slot,
+        const float* weights, int topk, const float* gate, const void* wd, float eps_d, const void* w, int wtype, float eps,
+        const int* rows, int R, void* out, float* out32, int H, const float* shift_w, float* shift_state,
+        const int* shift_slots, hipStream_t st);
 // elementwise.hip: a mixer input blended token by token with the row before; unit values mixed with another layer's
 int tq_token_shift(const float* x, const void* w, int wtype, float* state, const int* cu_seqlens, const int* slots,
         int B, void* out, int T, int H, hipStream_t st);

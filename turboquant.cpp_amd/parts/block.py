@@ -7,6 +7,8 @@ pass that normalises.
 """
 from __future__ import annotations
 
+import torch
+
 from .base import Part, register_part
 
 
@@ -128,10 +130,14 @@ class OutputNormBlock(Part):
             pending = None
         if self.mixer_shift is None:
             h, _ = ops.add_rmsnorm(x, pending, None, 0.0, ctx.act, stream=True)
-        else:       # the sum alone, then the blend with the row before from the float32 stream
-            if pending is not None:
-                ops.add_rmsnorm(x, pending, None, 0.0, ctx.act)
-            h = self.mixer_shift.forward(x, ctx, entry)
+        else:       # the sum alone, then the blend with the row before from the float32 stream; one launch where that can be
+            behind = self.mixer_shift.behind_sum(ctx, entry) if pending is not None and pending.weight.dtype == torch.float32 else None
+            if behind is not None:
+                h, _ = ops.add_rmsnorm(x, pending, None, 0.0, ctx.act, stream=True, shift=behind)
+            else:
+                if pending is not None:
+                    ops.add_rmsnorm(x, pending, None, 0.0, ctx.act)
+                h = self.mixer_shift.forward(x, ctx, entry)
         pending = ops.NormedDelta(self.mixer.forward(h, ctx, entry), self.mixer_norm.weight, self.mixer_norm.eps)
         if self.ffn is None:
             return pending
