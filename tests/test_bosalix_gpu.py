@@ -268,6 +268,22 @@ def test_slots_and_pages_used_again(made):
     assert all(v == 0 for v in eng.cache.pages_held().values())
 
 
+def test_a_prompt_longer_than_a_window_s_pool_runs_in_cuts(made):
+    """Where the pools of the groups with windows are sized for a window and a step of 128 positions, a prompt of 700 tokens
+    runs as six steps behind one call: the row that every layer keeps of the token before, the source layer's values of the
+    same step and the kept first positions all carry over from cut to cut."""
+    d, cfg, w = made("wide")
+    eng = engine_of(d, max_slots=1, window_step=128)
+    assert eng.cache.step_limit == 128
+    toks = tokens(cfg, 700, 13)
+    want = plain.forward(cfg, w, toks)
+    slot = eng.open(1)
+    got = eng.step(slot, [toks[:640]], [all_places(640)])
+    rows = [got] + [eng.step(slot, [toks[640:]], [all_places(60)])]
+    eng.close(slot)
+    check(torch.cat(rows), want, what="700 tokens in cuts of 128")
+
+
 def test_long_decoding_gives_pages_back_but_the_first(made):
     d, cfg, w = made("wide")
     eng = engine_of(d)

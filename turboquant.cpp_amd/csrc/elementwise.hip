@@ -1137,3 +1137,143 @@ TQ_API int tq_value_norm_mix(float* v, int64_t ld, int hd, int vd, int heads, fl
   TQ_LAUNCH_CHECK();
   return 0;
 }
+
+// ---------------------------------------------------------------- head norms, unit values, mix, rotation and cache write in one
+// What head_rmsnorm, value_norm_mix and rope_kv_write do one after the other, in one pass over a token's row: a wave takes a
+// head.  Query and key heads (qk_eps > 0): x * (1 / sqrt(sum(x^2) / norm_dim + qk_eps)) * w, w = wq or wk (null: heads of
+// that kind are left as they are), then the rotation; value heads (v_eps > 0): the head's first vd numbers divided by their
+// root mean square, then, with v_first, (1 - lambda) v + lambda v_first.  The values are also written back into qkv as the
+// cache holds them: for the tile write of whole runs of tokens that follows (write_kv 2), and for later layers that mix
+// them into their own.  The row holds every product's bias already.
+template <class W>
+__global__ __launch_bounds__(256) void attn_prep_kv_write_kernel(
+    float* __restrict__ qkv, int64_t ld, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+    const int* __restrict__ block_table, int bt_stride, const float* __restrict__ inv_freq, int pairing, int rot, float amp,
+    const W* __restrict__ wq, const W* __restrict__ wk, float qk_eps, int norm_dim, float v_eps, int vd,
+    const float* __restrict__ v_first, int64_t ld_first, int hd_first, const W* __restrict__ lambda,
+    act_t* __restrict__ q_out, act_t* __restrict__ k_pool, act_t* __restrict__ v_pool, int page_size, int64_t page_stride,
+    int nh, int nkv, int hd, int write_kv, int spb) {
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
+  const int heads = nh + 2 * nkv;
+  const int s0 = blockIdx.y * spb + wave, s1 = min(blockIdx.y * spb + spb, heads);
+  if (s0 >= s1) return;
+  const int pos = positions[t];
+  float* src_t = qkv + (size_t)t * ld;
+  act_t* q_t = q_out + (size_t)t * nh * hd;
+  act_t *k_t = nullptr, *v_t = nullptr;
+  if (write_kv && s1 > nh) {
+    const int page = block_table[(size_t)seq_of_token[t] * bt_stride + pos / page_size];
+    const int row = pos % page_size;
+    k_t = k_pool + (size_t)page * page_stride + (size_t)row * hd;
+    v_t = v_pool + (size_t)page * page_stride + row;
+  }
+  const int rot_end = write_kv ? min(s1, nh + nkv) : min(s1, nh);
+  const size_t kv_head_stride = (size_t)page_size * hd;
+  const int half = rot / 2;
+  float cs[4], sn[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = lane + TQ_WAVE * j;
+    cs[j] = 1.f;
+    sn[j] = 0.f;
+    if (i < half) {
+      sincosf((float)pos * inv_freq[i], &sn[j], &cs[j]);
+      sn[j] *= amp;
+      cs[j] *= amp;
+    }
+  }
+  for (int s = s0; s < rot_end; s += 4) {
+    const float* src = src_t + (size_t)s * hd;
+    act_t* dst = s < nh ? q_t + (size_t)s * hd : k_t + (size_t)(s - nh) * kv_head_stride;
+    const W* w = qk_eps > 0.f ? (s < nh ? wq : wk) : nullptr;
+    float rs = 1.0f;
+    if (w) {
+      float ss = 0.f;
+      for (int i = lane; i < hd; i += TQ_WAVE) ss = fmaf(src[i], src[i], ss);
+      rs = 1.0f / sqrtf(wave_sum(ss) / (float)norm_dim + qk_eps);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = lane + TQ_WAVE * j;
+      if (i < half) {
+        const int ia = pairing == 0 ? i : 2 * i;
+        const int ib = pairing == 0 ? i + half : 2 * i + 1;
+        float a = src[ia], b = src[ib];
+        if (w) {
+          a = a * rs * to_f32(w[ia]);
+          b = b * rs * to_f32(w[ib]);
+        }
+        dst[ia] = from_f32<act_t>(a * cs[j] - b * sn[j]);
+        dst[ib] = from_f32<act_t>(a * sn[j] + b * cs[j]);
+      }
+    }
+    for (int i = rot + lane; i < hd; i += TQ_WAVE) dst[i] = from_f32<act_t>(w ? src[i] * rs * to_f32(w[i]) : src[i]);
+  }
+  if (!write_kv) return;
+  const float lam = v_first ? to_f32(lambda[0]) : 0.f;
+  for (int s = s0; s < s1; s += 4) {
+    if (s < nh + nkv) continue;
+    const int g = s - nh - nkv;
+    float* src = src_t + (size_t)s * hd;
+    float r = 1.0f;
+    if (v_eps > 0.f) {
+      float ss = 0.f;
+      for (int i = lane; i < vd; i += TQ_WAVE) ss = fmaf(src[i], src[i], ss);
+      r = 1.0f / sqrtf(wave_sum(ss) / (float)vd + v_eps);
+    }
+    const float* fr = v_first ? v_first + (size_t)t * ld_first + (size_t)g * hd_first : nullptr;
+    act_t* col = v_t + (size_t)g * kv_head_stride;
+    for (int i = lane; i < hd; i += TQ_WAVE) {
+      float a = src[i];
+      if (i < vd) {
+        a *= r;
+        if (fr) a = (1.0f - lam) * a + lam * fr[i];
+        src[i] = a;
+      }
+      if (write_kv == 1) col[(size_t)i * page_size] = from_f32<act_t>(a);
+    }
+  }
+}
+
+// Arguments as tq_rope_kv_write_ex's (no bias: the rows hold it), with wq, wk (null: no norm of those heads), qk_eps,
+// norm_dim for the heads' norm before the rotation, v_eps (0: none) and vd for the values' unit norm, and v_first (null:
+// none), ld_first, hd_first, lambda for their mix.  hd at most 512 rotated numbers.
+TQ_API int tq_attn_prep_kv_write(float* qkv, int64_t ld, const int* positions, const int* seq_of_token, const int* block_table,
+                                 int bt_stride, const float* inv_freq, int pairing, int rot, float amp, const void* wq,
+                                 const void* wk, int wtype, float qk_eps, int norm_dim, float v_eps, int vd,
+                                 const float* v_first, int64_t ld_first, int hd_first, const void* lambda, void* q_out,
+                                 void* k_pool, void* v_pool, int page_size, int64_t page_stride, int T, int nh, int nkv,
+                                 int hd, int write_kv, const int* cu_seqlens, const int* slots, const int* start, int B,
+                                 int max_new, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (rot < 0 || rot % 2 != 0 || rot > hd || rot > 512 || (pairing != 0 && pairing != 1)) return TQ_ERR_BAD_ARG;
+  if (ld < (int64_t)(nh + 2 * nkv) * hd || norm_dim < 1 || norm_dim > hd || vd < 1 || vd > hd) return TQ_ERR_BAD_ARG;
+  if (v_first && (!lambda || vd > hd_first)) return TQ_ERR_BAD_ARG;
+  if (write_kv && (!k_pool || !v_pool)) return TQ_ERR_BAD_ARG;
+  constexpr int VEC = 16 / (int)sizeof(act_t);
+  const size_t vt_shmem = (size_t)hd * (VT_POS + VEC) * sizeof(act_t);
+  const bool tiles = write_kv && cu_seqlens && slots && start && B > 0 && B <= 65535 && nkv <= 65535 && max_new > 8 &&
+                     page_size % VT_POS == 0 && vt_shmem <= 64 * 1024;
+  if (tiles) write_kv = 2;
+  const int heads = nh + 2 * nkv;
+  int spb = 4;
+  while (spb < heads && (int64_t)T * ((heads + spb - 1) / spb) > 4096) spb *= 2;
+  if ((heads + spb - 1) / spb > 65535) return TQ_ERR_UNSUPPORTED;
+  TQ_DISPATCH_W(wtype, {
+    hipLaunchKernelGGL(attn_prep_kv_write_kernel<W>, dim3(T, (heads + spb - 1) / spb), dim3(256), 0, st, qkv, ld, positions,
+                       seq_of_token, block_table, bt_stride, inv_freq, pairing, rot, amp, (const W*)wq, (const W*)wk, qk_eps,
+                       norm_dim, v_eps, vd, v_first, ld_first, hd_first, (const W*)lambda, (act_t*)q_out, (act_t*)k_pool,
+                       (act_t*)v_pool, page_size, page_stride, nh, nkv, hd, write_kv, spb);
+  });
+  TQ_LAUNCH_CHECK();
+  if (tiles) {
+    if (vt_shmem > 48 * 1024)
+      (void)hipFuncSetAttribute((const void*)v_write_tile_kernel<VEC, 0>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)vt_shmem);
+    hipLaunchKernelGGL((v_write_tile_kernel<VEC, 0>), dim3((max_new + VT_POS - 1) / VT_POS + 1, nkv, B), dim3(256), vt_shmem, st,
+                       qkv, nullptr, cu_seqlens, slots, start, block_table, bt_stride, (act_t*)v_pool, page_size, page_stride,
+                       nh, nkv, hd, ld);
+    TQ_LAUNCH_CHECK();
+  }
+  return 0;
+}

@@ -73,6 +73,9 @@ _SIGNATURES = {
     "tq_token_shift": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr],
     "tq_value_norm_mix": [_c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_f32, _c_ptr, _c_i64, _c_int, _c_ptr, _c_int, _c_int,
                           _c_ptr],
+    "tq_attn_prep_kv_write": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_f32, _c_ptr, _c_ptr, _c_int,
+                              _c_f32, _c_int, _c_f32, _c_int, _c_ptr, _c_i64, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64,
+                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     "tq_act_rows": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "tq_gate_rows": [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "tq_latent_norm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_f32, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_ptr],
@@ -1503,6 +1506,73 @@ def value_norm_mix(v: torch.Tensor, num_heads: int, head_dim: int, value_dim: in
                                            first.stride(0) if first is not None else 0, fhd, _ptr(mix),
                                            _WTYPE[mix.dtype] if first is not None else 0, T, _stream()))
     return v
+
+
+def attn_prep_kv_write(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
+                       inv_freq: torch.Tensor, pairing: int, rotary_dim: int, k_pages: torch.Tensor | None,
+                       v_pages: torch.Tensor | None, layer_offset: int, page_size: int, page_stride: int, num_heads: int,
+                       num_kv_heads: int, head_dim: int, act, runs: dict | None = None, amplitude: float = 1.0,
+                       q_weight: torch.Tensor | None = None, k_weight: torch.Tensor | None = None, qk_eps: float = 0.0,
+                       norm_dim: int | None = None, value_eps: float = 0.0, value_dim: int | None = None,
+                       first: torch.Tensor | None = None, first_head_dim: int | None = None,
+                       mix: torch.Tensor | None = None) -> torch.Tensor:
+    """``head_rmsnorm``, ``value_norm_mix`` and ``rope_kv_write`` in one launch: every query and key head of the float32
+    rows ``qkv`` normed with its weights (``qk_eps`` > 0), every value head brought to unit root mean square over its first
+    ``value_dim`` numbers (``value_eps`` > 0) and mixed with ``first`` (as in ``value_norm_mix``), queries and keys rotated,
+    keys and values written into the pages; returns the queries.  The values are also written back into ``qkv`` as the
+    cache holds them.  ``qkv`` holds every product's bias already."""
+    k = "attn_prep_kv_write"
+    T = positions.numel()
+    width = (num_heads + 2 * num_kv_heads) * head_dim
+    _need(isinstance(qkv, torch.Tensor) and qkv.is_cuda and qkv.dtype == torch.float32 and tuple(qkv.shape) == (T, width)
+          and qkv.stride(1) == 1 and qkv.stride(0) >= width, k,
+          lambda: f"qkv must be float32 [{T}, {width}] on the GPU with unit stride along its rows")
+    _check(positions, k, "positions", torch.int32, (T,))
+    _check(seq_of_token, k, "seq_of_token", torch.int32, (T,))
+    _check(block_table, k, "block_table", torch.int32)
+    _need(block_table.dim() == 2, k, "block_table must be [B, pages]")
+    _check(inv_freq, k, "inv_freq", torch.float32)
+    _need(inv_freq.numel() * 2 == rotary_dim or rotary_dim == 0, k, lambda: f"inv_freq must hold rotary_dim/2 = {rotary_dim // 2} entries")
+    _need(rotary_dim <= 512 and qk_eps >= 0 and value_eps >= 0, k, "at most 512 rotated values; eps of 0 or more")
+    wtype = None
+    for name, w in (("q_weight", q_weight), ("k_weight", k_weight), ("mix", mix)):
+        if w is not None:
+            _check(w, k, name, tuple(_WTYPE), (1,) if name == "mix" else (head_dim,))
+            _need(wtype in (None, w.dtype), k, "the norms' weights and the mix must have one type")
+            wtype = w.dtype
+    vd = int(value_dim or head_dim)
+    fhd = 0
+    if first is not None:
+        fhd = int(first_head_dim or head_dim)
+        _need(first.is_cuda and first.dtype == torch.float32 and first.dim() == 2 and first.shape[0] == T
+              and first.shape[1] == num_kv_heads * fhd and first.stride(1) == 1 and vd <= fhd and mix is not None, k,
+              lambda: f"first must be float32 [{T}, {num_kv_heads * fhd}] on the GPU with unit stride along its rows, with a mix")
+    adt = ACT_DTYPES[dtype_name(act)]
+    q = torch.empty((T, num_heads * head_dim), dtype=adt, device=qkv.device)
+    write = k_pages is not None
+    kp = vp = None
+    if write:
+        _check(k_pages, k, "k_pages", adt)
+        _check(v_pages, k, "v_pages", adt)
+        _need(layer_offset + num_kv_heads * page_size * head_dim <= page_stride, k, "layer does not fit in a page")
+        esz = k_pages.element_size()
+        kp, vp = k_pages.data_ptr() + layer_offset * esz, v_pages.data_ptr() + layer_offset * esz
+    cu = slots = start = None
+    B = max_new = 0
+    if runs is not None and write and not runs["decode"]:
+        B = runs["slots"].numel()
+        cu, slots, start, max_new = runs["cu_seqlens"], runs["slots"], runs["start"], int(runs["max_new"])
+        _check(cu, k, "cu_seqlens", torch.int32, (B + 1,))
+        _check(slots, k, "slots", torch.int32, (B,))
+        _check(start, k, "start", torch.int32, (B,))
+        _need(int(runs["max_end"]) <= block_table.shape[1] * page_size, k, "positions reach beyond the page table")
+    _run(k, library(act).tq_attn_prep_kv_write(
+        _ptr(qkv), qkv.stride(0), _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], _ptr(inv_freq),
+        pairing, rotary_dim, float(amplitude), _ptr(q_weight), _ptr(k_weight), _WTYPE[wtype] if wtype is not None else 0,
+        float(qk_eps), int(norm_dim or head_dim), float(value_eps), vd, _ptr(first), first.stride(0) if first is not None else 0,
+        fhd, _ptr(mix), _ptr(q), kp, vp, page_size, page_stride, T, num_heads, num_kv_heads, head_dim, int(write), _ptr(cu),
+        _ptr(slots), _ptr(start), B, max_new, _stream()))
+    return q
 
 
 def latent_norm(src: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, copies: int, width: int, act) -> None:

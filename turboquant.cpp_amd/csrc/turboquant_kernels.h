@@ -206,6 +206,12 @@ int tq_token_shift(const float* x, const void* w, int wtype, float* state, const
         int B, void* out, int T, int H, hipStream_t st);
 int tq_value_norm_mix(float* v, int64_t ld, int hd, int vd, int heads, float eps, const float* first,
         int64_t ld_first, int hd_first, const void* lambda, int wtype, int T, hipStream_t st);
+int tq_attn_prep_kv_write(float* qkv, int64_t ld, const int* positions, const int* seq_of_token, const int* block_table,
+        int bt_stride, const float* inv_freq, int pairing, int rot, float amp, const void* wq, const void* wk, int wtype,
+        float qk_eps, int norm_dim, float v_eps, int vd, const float* v_first, int64_t ld_first, int hd_first,
+        const void* lambda, void* q_out, void* k_pool, void* v_pool, int page_size, int64_t page_stride, int T, int nh,
+        int nkv, int hd, int write_kv, const int* cu_seqlens, const int* slots, const int* start, int B, int max_new,
+        hipStream_t st);
 // sampling.hip: greedy choice, negative log-likelihood, repetition penalty, temperature and top-p (both libraries; the two *_static entry points are declared in no_alloc.h)
 int tq_argmax(const float* logits, int R, int V, int* out, hipStream_t st);
 int tq_nll(const float* logits, int R, int V, const int* target, float* out, hipStream_t st);

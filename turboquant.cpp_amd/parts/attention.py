@@ -272,6 +272,23 @@ class GroupedQueryAttention(Part):
         proj = ops.gemm(normed, self.qkv_weight, ctx.act, bias=self.qkv_bias)
         width = (H + 2 * G) * D
         qkv = proj[:, :width]
+        if (self.value_norm_eps is not None or self.value_mix is not None) and kv.owns and self.rotated_norm_eps is None:
+            # head norms, unit values and their mix, rotation and cache write: one pass over a token's row
+            first, first_dim = b.scratch[("value_mix",)] if self.value_mix == "mix" else (None, None)
+            q = ops.attn_prep_kv_write(qkv, b.positions, b.slot_of_token, kv.table, self.position.table(ctx.device),
+                                       self.position.pairing_code, self.position.rotary_dim, kv.k_pages, kv.v_pages,
+                                       kv.layer_offset, kv.page_size, kv.page_stride, H, G, D, ctx.act, runs=b.runs(),
+                                       amplitude=amplitude, q_weight=self.q_norm, k_weight=self.k_norm,
+                                       qk_eps=self.qk_norm_eps or 0.0, norm_dim=self.key_dim,
+                                       value_eps=self.value_norm_eps or 0.0, value_dim=self.value_dim, first=first,
+                                       first_head_dim=first_dim, mix=self.mix if first is not None else None)
+            if self.value_mix == "source":
+                b.scratch[("value_mix",)] = (qkv[:, (H + G) * D:], D)
+            o = ops.attention(q, kv.k_pages, kv.v_pages, kv.layer_offset, b.positions, b.slot_of_token, kv.table,
+                              kv.page_size, kv.page_stride, H, self.num_kv_heads, D, self.window, self.scale, ctx.act,
+                              runs=b.runs(), head_gate=proj[:, width:width + H] if self.has_head_gate else None,
+                              **self._score_options())
+            return ops.gemm(o, self.out_weight, ctx.act, bias=self.out_bias, partial_sums=True)
         if self.qk_norm_eps is not None:
             if proj.shape[1] != width:
                 raise ValueError("the norm of the heads before the rotation does not go with a gate per head")
