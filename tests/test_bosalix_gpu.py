@@ -517,6 +517,58 @@ def test_unit_values_and_their_mix():
         assert np.abs(got - want).max() < 2e-6
 
 
+def test_head_norms_unit_values_rotation_and_cache_write_in_one_launch():
+    """``attn_prep_kv_write`` against ``head_rmsnorm``, ``value_norm_mix`` and ``rope_kv_write`` one after the other: the same
+    queries, the same pages, the same values left behind in the rows; a prompt's run and single decoded tokens."""
+    from turboquant_cpp_amd.csrc import ops
+    rng = np.random.default_rng(5)
+    nh, nkv, hd, kd, vd, page, extra = 6, 2, 48, 40, 24, 64, 5
+    width = (nh + 2 * nkv) * hd
+    inv_freq = f32(1.0 / 100.0 ** (np.arange(8) / 8.0))
+    for act in ("float32", "bfloat16"):
+        adt = torch.float32 if act == "float32" else torch.bfloat16
+        wq, wk = (torch.tensor(np.concatenate([1 + 0.2 * rng.standard_normal(kd), np.zeros(hd - kd)]), dtype=adt, device="cuda") for _ in range(2))
+        mix = torch.tensor([0.3], dtype=adt, device="cuda")
+        for pairing in (0, 1):
+            for n_new, start, with_first in ((70, 0, False), (70, 30, True), (3, 200, True), (1, 64, False)):
+                T = n_new
+                rows = rng.standard_normal((T, width + extra))
+                rows[:, :width].reshape(T, nh + 2 * nkv, hd)[:, :nh + nkv, kd:] = 0.0      # heads laid out wider hold zeros
+                rows[:, :width].reshape(T, nh + 2 * nkv, hd)[:, nh + nkv:, vd:] = 0.0
+                first = f32(rng.standard_normal((T, nkv * 32))) if with_first else None
+                positions = torch.arange(start, start + T, dtype=torch.int32, device="cuda")
+                seq = torch.full((T,), 1, dtype=torch.int32, device="cuda")
+                n_pages = -(-(start + T) // page)
+                table = torch.full((2, n_pages), -1, dtype=torch.int32, device="cuda")
+                table[1] = torch.tensor(rng.permutation(n_pages), dtype=torch.int32)
+                stride = 2 * nkv * page * hd                        # two layers to a page; this one is the second
+                offset = nkv * page * hd
+                decode = T == 1
+                runs = {"cu_seqlens": torch.tensor([0, T], dtype=torch.int32, device="cuda"), "slots": torch.tensor([1], dtype=torch.int32, device="cuda"),
+                        "start": torch.tensor([start], dtype=torch.int32, device="cuda"), "max_new": T, "max_end": start + T, "decode": decode}
+                results = []
+                for fused in (False, True):
+                    t = f32(rows)
+                    qkv = t[:, :width]
+                    kp = torch.zeros((n_pages * stride,), dtype=adt, device="cuda")
+                    vp = torch.zeros_like(kp)
+                    args = (positions, seq, table, inv_freq, pairing, 16, kp, vp, offset, page, stride, nh, nkv, hd, act)
+                    if fused:
+                        q = ops.attn_prep_kv_write(qkv, *args, runs=runs, q_weight=wq, k_weight=wk, qk_eps=1e-5, norm_dim=kd,
+                                                   value_eps=1e-5, value_dim=vd, first=first, first_head_dim=32,
+                                                   mix=mix if with_first else None)
+                    else:
+                        ops.head_rmsnorm(qkv, wq, wk, 1e-5, nh, nkv, hd, act, norm_dim=kd)
+                        ops.value_norm_mix(qkv[:, (nh + nkv) * hd:], nkv, hd, vd, 1e-5, act, first=first, first_head_dim=32,
+                                           mix=mix if with_first else None)
+                        q = ops.rope_kv_write(qkv, *args, runs=runs)
+                    results.append((q.float(), kp.float(), vp.float(), t[:, (nh + nkv) * hd:].clone()))
+                tol = 2e-6 if act == "float32" else 1e-2
+                for name, x, y in zip(("queries", "key pages", "value pages", "values left in the rows"), *results):
+                    assert (x - y).abs().max() <= tol * max(1.0, float(y.abs().max())), (act, pairing, n_new, start, name)
+                assert float(results[1][1].abs().max()) > 0 and float(results[1][2].abs().max()) > 0
+
+
 def test_choice_by_corrected_scores_with_identity_experts():
     from turboquant_cpp_amd.csrc import ops
     rng = np.random.default_rng(2)
