@@ -522,7 +522,7 @@ def test_head_norms_unit_values_rotation_and_cache_write_in_one_launch():
     queries, the same pages, the same values left behind in the rows; a prompt's run and single decoded tokens."""
     from turboquant_cpp_amd.csrc import ops
     rng = np.random.default_rng(5)
-    nh, nkv, hd, kd, vd, page, extra = 6, 2, 48, 40, 24, 64, 5
+    nh, nkv, hd, kd, vd, page, extra = 6, 2, 48, 40, 24, 64, 0
     width = (nh + 2 * nkv) * hd
     inv_freq = f32(1.0 / 100.0 ** (np.arange(8) / 8.0))
     for act in ("float32", "bfloat16"):
